@@ -2,14 +2,18 @@
 HIPCC ?= /opt/rocm/bin/hipcc
 ARCH  ?= gfx950
 CSRC  := vllm_omni_draft_amd/csrc
-SRCS  := $(CSRC)/sd_runtime.hip $(CSRC)/sd_sampling.hip $(CSRC)/sd_linear.hip $(CSRC)/sd_linear_wide.hip $(CSRC)/sd_attention.hip $(CSRC)/sd_ipc.hip $(CSRC)/sd_chain.hip $(CSRC)/sd_draft_layer.hip
+SRCS  := $(CSRC)/sd_base.hip $(CSRC)/sd_runtime.hip $(CSRC)/sd_sampling.hip $(CSRC)/sd_linear.hip $(CSRC)/sd_linear_wide.hip $(CSRC)/sd_attention.hip $(CSRC)/sd_ipc.hip $(CSRC)/sd_chain.hip $(CSRC)/sd_draft_layer.hip $(CSRC)/sd_seqmix.hip
 OBJS  := $(SRCS:.hip=.o)
 LIB   := vllm_omni_draft_amd/libsd_amd.so
 EXTRA ?=
 # -ffp-contract=off: whether a*b+c becomes one fma is otherwise the compiler's choice per
 # template instantiation, and two instantiations of a kernel (one or two token tiles, ring
 # depths, ...) must give a row the same bits.
-FLAGS := --offload-arch=$(ARCH) -O3 -std=c++17 -fPIC -ffp-contract=off -Wall -Wno-unused-function $(EXTRA)
+# -packed-fp32-ops off: the compiler forms packed f32 instructions from scalar code by itself, and
+# some of their forms have given wrong results on this hardware pool; the host pass warns that it
+# does not know the feature, which is harmless.
+FLAGS := --offload-arch=$(ARCH) -O3 -std=c++17 -fPIC -ffp-contract=off -Wall -Wno-unused-function \
+	-Xclang -target-feature -Xclang -packed-fp32-ops $(EXTRA)
 
 # The CPU build of the same C ABI (C++ / OpenMP): its own library, loaded only when the host
 # code is told to (SD_AMD_BACKEND=cpu); the GPU library never falls back to it.
@@ -26,6 +30,15 @@ $(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/sd_common.h include/sd_amd.h
 
 $(LIB): $(OBJS)
 	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(OBJS) -L/opt/rocm/lib -lrccl -Wl,-rpath,/opt/rocm/lib
+
+# The part of the library that layer-list models (sequence mixers, sampling) need, for a first
+# run in a fresh checkout that should not wait for every kernel family to compile.  The package
+# loads it only where the whole library has not been built.
+SEQ_LIB  := vllm_omni_draft_amd/libsd_seq.so
+SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_sampling.o
+$(SEQ_LIB): $(SEQ_OBJS)
+	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(SEQ_OBJS)
+seq: $(SEQ_LIB)
 
 # Diagnostic build with in-kernel timestamps (experiments/*_stamps.py load it through SD_AMD_LIB);
 # never loaded by the package on its own.
@@ -51,7 +64,7 @@ $(SWITCH_LIB): $(OBJS)
 wide-switch: $(SWITCH_LIB)
 
 clean:
-	rm -f $(OBJS) $(LIB) $(CPU_LIB)
+	rm -f $(OBJS) $(LIB) $(CPU_LIB) $(SEQ_LIB)
 	rm -rf $(STAMP_DIR) build/exp/*.o build/exp/*.so
 
-.PHONY: all clean stamps wide-switch
+.PHONY: all clean stamps wide-switch seq

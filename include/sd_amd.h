@@ -1023,6 +1023,143 @@ int sd_graph_end(sd_stream_t stream, sd_graph** out);
 int sd_graph_launch(sd_graph* g, sd_stream_t stream);
 void sd_graph_destroy(sd_graph* g);
 
+/* ------------------------------------------------------------------------
+ * Sequence mixers beyond softmax attention, and decoders built from a list of layers
+ * (no counterpart in the reference tree or upstream's speculative path: recurrent and
+ * windowed layers as hybrid language models use them).
+ *
+ * Activations are f32 buffers.  `w_f32` / `cache_f32` say whether a weight or cache pointer
+ * holds f32 or bf16 elements; with bf16 weights the operands of matrix products are rounded to
+ * bf16 values (f32 accumulation), with f32 weights nothing is.  A ragged batch is a list of token
+ * rows, each with its position in its sequence (row_pos) and its sequence slot (row_slot), and a
+ * list of entries {slot, first row, rows, first position}: one run of consecutive tokens of one
+ * sequence.  Every result element is summed in an order fixed by its own position, so a token's
+ * bits do not depend on the batch around it or on how its prompt was cut.
+ * ---------------------------------------------------------------------- */
+
+/* y[M, N] = x[M, K] w[N, K]^T + bias[N] (bias may be NULL).  x2 != NULL: the operand is
+ * relu(x) * x2 (a gated feed-forward's activation; same ldx).  w row-major, any N and K.   */
+int sd_matmul_rows(const float* x, const float* x2, int64_t ldx, const void* w, int w_f32,
+                   const float* bias, float* y, int64_t ldy, int M, int N, int K,
+                   sd_stream_t stream);
+/* out[i] = x[rows ? rows[i] : i] / sqrt(mean(x^2) + eps) * (offset + w): offset 1 for a weight
+ * stored around zero, 0 for a plain weight.                                                */
+int sd_rmsnorm_rows(const float* x, const int32_t* rows, const void* w, int w_f32, float offset,
+                    float eps, float* out, int n, int W, sd_stream_t stream);
+/* Per (row, head), in place on q [rows, Hq*dk] and k [rows, Hk*dk] (row stride ld): rotary
+ * embedding of the first rot_dims channels (rot_layout 0: channel i pairs with i + rot_dims/2;
+ * 1: channel 2i with 2i+1; angle row_pos * inv_freq[i], inv_freq f64 [rot_dims/2]), then a
+ * division by the vector's root mean square (unit_norm), then q_scale / k_scale.  With a cache
+ * (k_cache != NULL) the finished keys and the value rows v [rows, Hk*dv] are appended to pages
+ * of `page` tokens: row (page, head, token) of dk / dv elements.                            */
+int sd_head_prep(float* q, float* k, const float* v, int64_t ld, const int32_t* row_pos,
+                 const int32_t* row_slot, int n_rows, int Hq, int Hk, int dk, int dv,
+                 int rot_dims, int rot_layout, const double* inv_freq, int unit_norm, float eps,
+                 float q_scale, float k_scale, void* k_cache, void* v_cache, int cache_f32,
+                 const int32_t* block_tables, int max_blocks, int page, sd_stream_t stream);
+/* out[r, c] = sigmoid(z[r, c])^(1/tau), through the logarithm.                              */
+int sd_sigmoid_power(const float* z, int64_t ldz, float tau, float* out, int n_rows, int n_cols,
+                     sd_stream_t stream);
+/* Decayed outer-product recurrence, token by token for every entry and head:
+ *   S <- diag(d_t) S + k_t v_t^T,   o_t = S^T q_t,
+ * S [dk, dv] f32 in state [slots, H, dk, dv] (taken as zero for an entry that starts at
+ * position 0, written back at the end).  q, k [rows, H*dk], v [rows, H*dv] with row stride ld;
+ * decay: per_channel ? [rows, H*dk] : [H].  out [rows, H*dv].  dk <= 256.                  */
+int sd_decay_scan(const float* q, const float* k, const float* v, int64_t ld, const float* decay,
+                  int per_channel, float* state, const int32_t* entries, int n_entries,
+                  float* out, int H, int dk, int dv, sd_stream_t stream);
+/* y = o * (unit_norm ? 1/rms(o over the head) : 1) * (norm_w ? norm_w[c] : 1) * gate(g);
+ * gate_kind 0: g*sigmoid(g), 1: sigmoid(g).  o, y [rows, H*dv]; g row stride ldg.            */
+int sd_head_post(const float* o, const float* g, int64_t ldg, const void* norm_w, int w_f32,
+                 int unit_norm, float eps, int gate_kind, float* y, int n_rows, int H, int dv,
+                 int round_bf16_out, sd_stream_t stream);
+/* Pooled entries a page of the pooled caches holds (blocks of `pool` tokens ending in it). */
+int sd_pooled_slots_per_page(int page, int pool);
+/* Sliding-window attention with pooled blocks and sigmoid weights over the cache sd_head_prep
+ * fills.  Row at position i sees tokens j with 0 <= i - j < window, and block b (tokens
+ * b*pool .. b*pool+pool-1) once b*pool + pool - 1 <= i - window, as the mean of its cached keys
+ * and of its values (pk_cache / pv_cache, f32, sd_pooled_slots_per_page entries per page and
+ * head; computed here when a row completes a block).  out[r, h] = sum over visible keys of
+ * sigmoid(q.k * scale + head_bias[h]) * v; query head h reads kv head h / (H/G).  dv <= 256. */
+int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                             int cache_f32, float* pk_cache, float* pv_cache,
+                             const int32_t* row_pos, const int32_t* row_slot,
+                             const int32_t* block_tables, int max_blocks, int page, int n_rows,
+                             int H, int G, int dk, int dv, int window, int pool, float scale,
+                             const float* head_bias, float* out, sd_stream_t stream);
+/* x += sigmoid(z1) * a + sigmoid(z2) * b (b, z2 may be NULL); x, a, b [rows, W].            */
+int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* a,
+                      const float* b, int n_rows, int W, sd_stream_t stream);
+
+typedef enum {
+  SD_MIX_HEAD_DECAY = 0,    /* recurrence with a fixed decay per head (retention) */
+  SD_MIX_CHANNEL_DECAY = 1, /* recurrence with an input-dependent decay per key channel */
+  SD_MIX_WINDOW_POOL = 2    /* sd_window_pool_attention */
+} sd_mixer_kind;
+
+/* One layer: h = norm(x); x += sigmoid(r1) * mixer(h) + sigmoid(r2) * ff(h).  w_in stacks every
+ * matrix that reads h, rows in this order: q [heads*dim], k [kv_heads*dim], v [kv_heads*vdim],
+ * g [heads*vdim], r1 [width], r2 [width] and the feed-forward's gate [ff], up [ff] (if ff > 0),
+ * a1 [rank] (channel decay); b_in is its f32 bias.                                         */
+typedef struct {
+  int kind;
+  int heads, kv_heads, dim, vdim;
+  int ff;                  /* 0: the layer has no feed-forward */
+  int rot_dims, rot_layout;
+  const double* inv_freq;  /* [rot_dims/2] device, or NULL */
+  int qk_unit_norm;
+  float q_scale, k_scale, score_scale;
+  int window, pool;
+  int rank;
+  float tau;
+  const void* norm_w;      /* [width], stored around zero */
+  const void* w_in;
+  const float* b_in;
+  const void* w_o;         /* [width, heads*vdim] */
+  const void* w_down;      /* [width, ff] or NULL */
+  const void* w_a2;        /* [heads*dim, rank] or NULL */
+  const float* b_a2;
+  const float* head_decay; /* [heads] or NULL */
+  const float* head_bias;  /* [heads] or NULL */
+  const void* head_norm_w; /* [vdim] plain weight of the per-head output norm, or NULL */
+  float* state;            /* recurrent: [slots, heads, dim, vdim] */
+  void* k_cache;           /* window attention: pages, see sd_head_prep */
+  void* v_cache;
+  float* pk_cache;
+  float* pv_cache;
+} sd_seq_layer;
+
+typedef struct {
+  int n_layers, width, vocab;
+  int weights_f32;         /* element type of every weight and of the k / v caches */
+  float norm_eps;
+  const void* embed;       /* [vocab, width]; also the output head */
+  const void* final_norm_w;
+  const sd_seq_layer* layers; /* copied */
+} sd_seq_model_desc;
+
+typedef struct {
+  int n_rows, n_entries;
+  const int32_t* tokens;   /* [n_rows] */
+  const int32_t* row_pos;  /* [n_rows] */
+  const int32_t* row_slot; /* [n_rows] */
+  const int32_t* entries;  /* [n_entries][4] */
+  const int32_t* block_tables; /* [slots, max_blocks] pages of each slot (window layers) */
+  int max_blocks, page;
+  int n_out;
+  const int32_t* out_rows; /* [n_out] rows whose logits are wanted */
+  float* logits;           /* [n_out, vocab] */
+  float* layer_out;        /* NULL, or [n_layers, n_rows, width]: the residual after each layer */
+} sd_seq_batch;
+
+typedef struct sd_seq_model sd_seq_model;
+sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc);
+void sd_seq_model_destroy(sd_seq_model* m);
+size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out);
+/* One pass over a ragged batch: enqueues kernels only.                                     */
+int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* batch, void* workspace,
+                         size_t workspace_bytes, sd_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,7 +10,11 @@ import os
 from typing import Optional
 
 _LIB_NAME = "libsd_amd.so"
+# The sources that layer-list models need, built alone (`make seq`): loaded where the whole
+# library has not been built (a first run in a fresh checkout); it exports a subset of the ABI.
+_SEQ_LIB_NAME = "libsd_seq.so"
 _lib: Optional[C.CDLL] = None
+_partial = False
 
 c_i32p = C.POINTER(C.c_int32)
 vp = C.c_void_p
@@ -69,6 +73,28 @@ class RowAdds(C.Structure):
 
 class RopePositions(C.Structure):
     _fields_ = [("pos", vp), ("delta", vp), ("section_t", i32), ("section_h", i32)]
+
+
+class SeqLayer(C.Structure):
+    """sd_seq_layer"""
+    _fields_ = [("kind", i32), ("heads", i32), ("kv_heads", i32), ("dim", i32), ("vdim", i32), ("ff", i32),
+                ("rot_dims", i32), ("rot_layout", i32), ("inv_freq", vp), ("qk_unit_norm", i32),
+                ("q_scale", C.c_float), ("k_scale", C.c_float), ("score_scale", C.c_float),
+                ("window", i32), ("pool", i32), ("rank", i32), ("tau", C.c_float),
+                ("norm_w", vp), ("w_in", vp), ("b_in", vp), ("w_o", vp), ("w_down", vp), ("w_a2", vp),
+                ("b_a2", vp), ("head_decay", vp), ("head_bias", vp), ("head_norm_w", vp), ("state", vp),
+                ("k_cache", vp), ("v_cache", vp), ("pk_cache", vp), ("pv_cache", vp)]
+
+
+class SeqModelDesc(C.Structure):
+    _fields_ = [("n_layers", i32), ("width", i32), ("vocab", i32), ("weights_f32", i32),
+                ("norm_eps", C.c_float), ("embed", vp), ("final_norm_w", vp), ("layers", C.POINTER(SeqLayer))]
+
+
+class SeqBatch(C.Structure):
+    _fields_ = [("n_rows", i32), ("n_entries", i32), ("tokens", vp), ("row_pos", vp), ("row_slot", vp),
+                ("entries", vp), ("block_tables", vp), ("max_blocks", i32), ("page", i32), ("n_out", i32),
+                ("out_rows", vp), ("logits", vp), ("layer_out", vp)]
 
 
 # name -> (restype, argtypes); every symbol include/sd_amd.h declares.
@@ -182,6 +208,21 @@ SIGNATURES = {
     "sd_graph_begin": (i32, [vp]),
     "sd_graph_end": (i32, [vp, C.POINTER(vp)]),
     "sd_graph_launch": (i32, [vp, vp]),
+    "sd_matmul_rows": (i32, [vp, vp, i64, vp, i32, vp, vp, i64, i32, i32, i32, vp]),
+    "sd_rmsnorm_rows": (i32, [vp, vp, vp, i32, C.c_float, C.c_float, vp, i32, i32, vp]),
+    "sd_head_prep": (i32, [vp, vp, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, i32, C.c_float,
+                           C.c_float, C.c_float, vp, vp, i32, vp, i32, i32, vp]),
+    "sd_sigmoid_power": (i32, [vp, i64, C.c_float, vp, i32, i32, vp]),
+    "sd_decay_scan": (i32, [vp, vp, vp, i64, vp, i32, vp, vp, i32, vp, i32, i32, i32, vp]),
+    "sd_head_post": (i32, [vp, vp, i64, vp, i32, i32, C.c_float, i32, vp, i32, i32, i32, i32, vp]),
+    "sd_pooled_slots_per_page": (i32, [i32, i32]),
+    "sd_window_pool_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
+                                       i32, i32, i32, C.c_float, vp, vp, vp]),
+    "sd_gated_residual": (i32, [vp, vp, vp, i64, vp, vp, i32, i32, vp]),
+    "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
+    "sd_seq_model_destroy": (None, [vp]),
+    "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32]),
+    "sd_seq_model_forward": (i32, [vp, C.POINTER(SeqBatch), vp, C.c_size_t, vp]),
     "sd_graph_destroy": (None, [vp]),
 }
 
@@ -206,7 +247,8 @@ def lib_path() -> str:
     override = os.environ.get("SD_AMD_LIB")
     if override:
         return os.path.abspath(override)
-    return os.path.join(here, _LIB_NAME)
+    full, seq = os.path.join(here, _LIB_NAME), os.path.join(here, _SEQ_LIB_NAME)
+    return seq if (not os.path.exists(full) and os.path.exists(seq)) else full
 
 
 def load() -> C.CDLL:
@@ -218,13 +260,33 @@ def load() -> C.CDLL:
     if not os.path.exists(path):
         raise SdError(f"{path} is missing: build it with `make` (hipcc --offload-arch=gfx950; "
                       "g++ for the CPU build); nothing falls back to another library or to PyTorch")
+    global _partial
     lib = C.CDLL(path)
+    _partial = os.path.basename(path) == _SEQ_LIB_NAME
     for name, (res, args) in SIGNATURES.items():
+        if _partial and not hasattr(lib, name):
+            continue             # the subset build: calling such an entry point raises AttributeError
         fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported
         fn.restype = res
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+def ensure_built(seq_only: bool = False) -> str:
+    """Builds the GPU library in-tree if no build of it is there (hipcc, gfx950) and returns the
+    path that load() will open.  seq_only: only what layer-list models need, unless the whole
+    library exists already."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    if backend() == "gpu" and not os.environ.get("SD_AMD_LIB"):
+        full, seq = os.path.join(here, _LIB_NAME), os.path.join(here, _SEQ_LIB_NAME)
+        if not os.path.exists(full) and not (seq_only and os.path.exists(seq)):
+            import subprocess
+            jobs = str(min(16, os.cpu_count() or 4))
+            subprocess.run(["make", "-C", os.path.dirname(here), "-j" + jobs,
+                            os.path.relpath(seq if seq_only else full, os.path.dirname(here))],
+                           check=True, stdout=subprocess.DEVNULL)
+    return lib_path()
 
 
 def last_error() -> str:

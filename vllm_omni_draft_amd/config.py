@@ -11,7 +11,7 @@ import math
 import os
 import dataclasses
 from dataclasses import dataclass, field, fields
-from typing import Optional
+from typing import List, Optional
 
 import torch
 
@@ -206,3 +206,165 @@ def rope_table(cfg: ModelConfig, device="cpu") -> torch.Tensor:
             raise ValueError(f"rope scaling {kind!r} not supported")
     ang = torch.arange(cfg.max_pos, dtype=torch.float32)[:, None] * inv.float()[None, :]
     return torch.cat([ang.cos(), ang.sin()], dim=1).contiguous().to(device)
+
+
+# ---------------------------------------------------------------------------------------------
+# Decoders described layer by layer (recurrent and windowed mixers); served by seq_engine.SeqEngine.
+MIXER_KINDS = ("retention", "gla", "attention")
+
+
+@dataclass
+class MixerSpec:
+    """One layer's token mixer.  kind "retention": decayed linear attention with a fixed decay per
+    head and rotate-half rotary positions; "gla": decayed linear attention whose decay per key
+    channel comes from the input through a low-rank pair of matrices (sigmoid(z)^(1/tau));
+    "attention": grouped-query attention over a sliding window plus mean-pooled blocks of the
+    tokens before it, with sigmoid weights, interleaved rotary positions and unit-norm q / k."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0              # 0: as many as heads
+    rot_dims: int = 0              # leading channels of a head that are rotated (0: none)
+    rot_base: float = 10000.0
+    rot_layout: str = "half"       # "half": channel i pairs with i + rot_dims/2; "interleaved": 2i with 2i+1
+    decay: Optional[tuple] = None  # retention: one factor per head
+    tau: float = 1.0               # gla
+    rank: int = 0                  # gla: inner size of the low-rank pair (a tensor's shape gives it)
+    scale: float = 1.0             # attention: factor of the scores
+    window: int = 0                # attention: tokens seen, the current one included
+    pool: int = 1                  # attention: tokens per pooled block
+
+    def validate(self) -> None:
+        if self.kind not in MIXER_KINDS:
+            raise ValueError(f"unknown mixer {self.kind!r}; known: {MIXER_KINDS}")
+        self.kv_heads = self.kv_heads or self.heads
+        if min(self.heads, self.kv_heads, self.dim, self.vdim) < 1 or self.heads % self.kv_heads:
+            raise ValueError(f"mixer sizes: heads {self.heads}, kv_heads {self.kv_heads}, dim {self.dim}, "
+                             f"vdim {self.vdim}")
+        if self.rot_layout not in ("half", "interleaved"):
+            raise ValueError(f"unknown rotary layout {self.rot_layout!r}")
+        if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.dim:
+            raise ValueError(f"rot_dims {self.rot_dims} must be even and at most dim {self.dim}")
+        if self.kind == "attention":
+            if self.window < 1 or self.pool < 1:
+                raise ValueError("an attention mixer needs window >= 1 and pool >= 1")
+            if self.vdim > 256:
+                raise ValueError("attention vdim above 256 is not supported")
+        else:
+            if self.kv_heads != self.heads:
+                raise ValueError("a recurrent mixer has one key head per query head")
+            if self.dim > 256:
+                raise ValueError("recurrent key size above 256 is not supported")
+        if self.kind == "retention":
+            if self.decay is None or len(self.decay) != self.heads:
+                raise ValueError("retention needs one decay per head")
+            self.decay = tuple(float(d) for d in self.decay)
+        if self.kind == "gla" and not self.tau > 0:
+            raise ValueError("gla needs tau > 0")
+
+
+@dataclass
+class SeqLayerSpec:
+    mixer: MixerSpec
+    ff: int = 0                    # width of the gated feed-forward beside the mixer; 0: none
+
+
+@dataclass
+class SeqModelConfig:
+    """A decoder as a list of layers.  Every layer is  h = norm(x);  x += sigmoid(R1 h + r1) *
+    mixer(h) + sigmoid(R2 h + r2) * ff(h)  with an RMS norm whose weight is stored around zero;
+    the output head is the embedding table."""
+    arch: str
+    width: int
+    vocab: int
+    layers: List["SeqLayerSpec"]
+    norm_eps: float = 1e-5
+    name: str = "custom"
+
+    def validate(self) -> None:
+        if self.width < 1 or self.vocab < 1 or not self.layers:
+            raise ValueError("a model needs width, vocab and at least one layer")
+        for l in self.layers:
+            l.mixer.validate()
+            if l.ff < 0:
+                raise ValueError("ff must be >= 0")
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    def param_count(self) -> int:
+        W, n = self.width, self.vocab * self.width + self.width
+        for l in self.layers:
+            m = l.mixer
+            n += W + W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim) + 2 * m.heads * m.vdim) + W * W + W
+            n += (m.rank * (W + m.heads * m.dim) + m.heads * m.dim + m.vdim) if m.kind == "gla" else 0
+            n += (3 * l.ff * W + W * W + W) if l.ff else 0
+        return n
+
+    def state_bytes_per_seq(self) -> int:
+        return sum(4 * l.mixer.heads * l.mixer.dim * l.mixer.vdim for l in self.layers
+                   if l.mixer.kind != "attention")
+
+
+def puguzen_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides) -> SeqModelConfig:
+    """A Puguzen config.json.  tensor_shapes (name -> shape) supplies the sizes the file does not
+    state (the inner size of a gla layer's low-rank pair)."""
+    layers = []
+    for i, l in enumerate(cfg["layers"]):
+        m, kind = l["mixer"], l["type"]
+        rot, mask = m.get("rot") or {}, m.get("mask") or {}
+        rank = 0
+        if kind == "gla":
+            shape = (tensor_shapes or {}).get(f"l{i}.mix.a1")
+            rank = int(shape[0]) if shape is not None else int(m.get("rank", 0))
+        spec = MixerSpec(kind=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         kv_heads=int(m.get("kv_heads", 0)), rot_dims=int(rot.get("dims", 0)),
+                         rot_base=float(rot.get("base", 10000.0)),
+                         rot_layout="interleaved" if kind == "attention" else "half",
+                         decay=tuple(m["decay"]) if "decay" in m else None, tau=float(m.get("tau", 1.0)),
+                         rank=rank, scale=float(m.get("scale", 1.0)), window=int(mask.get("size", 0)),
+                         pool=int(mask.get("pool", 1)))
+        mlp = l.get("mlp")
+        if mlp and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported")
+        layers.append(SeqLayerSpec(spec, int(mlp["ff"]) if mlp else 0))
+    out = SeqModelConfig(arch="puguzen", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers,
+                         norm_eps=float(cfg["norm"]["eps"]), name=cfg.get("architecture", "Puguzen"))
+    for k, v in overrides.items():
+        if not hasattr(out, k):
+            raise ValueError(f"Unknown config parameter: {k}")
+        setattr(out, k, v)
+    out.validate()
+    return out
+
+
+# config.json "architecture" -> builder of a layer-list config
+SEQ_ARCHITECTURES = {"Puguzen": puguzen_config}
+
+
+def safetensors_shapes(path: str) -> dict:
+    """name -> shape from a safetensors file's header (8-byte length, then JSON)."""
+    import struct
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        head = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in head.items() if k != "__metadata__"}
+
+
+def load_model_config(model_dir: str, **overrides):
+    """The configuration class a checkpoint folder asks for: a layer-list model if its
+    config.json names one of SEQ_ARCHITECTURES, else a Hugging Face decoder (ModelConfig)."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    arch = cfg.get("architecture")
+    if arch in SEQ_ARCHITECTURES:
+        shapes = {}
+        for fn in sorted(os.listdir(model_dir)):
+            if fn.endswith(".safetensors"):
+                shapes.update(safetensors_shapes(os.path.join(model_dir, fn)))
+        return SEQ_ARCHITECTURES[arch](cfg, shapes, **overrides)
+    if arch is not None and "model_type" not in cfg:
+        raise ValueError(f"unknown architecture {arch!r}; known: {sorted(SEQ_ARCHITECTURES)}")
+    return from_hf_config(cfg, **overrides)

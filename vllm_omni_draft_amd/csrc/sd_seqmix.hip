@@ -1,0 +1,775 @@
+// Sequence mixers beyond softmax attention, for decoders whose layers are listed one by one
+// (sd_seq_model): decayed linear-attention recurrences (a fixed decay per head, or a decay per
+// key channel computed from the input), sliding-window attention with pooled blocks and sigmoid
+// weights, offset RMS norms, partial rotary embeddings in both pair layouts, gated residuals.
+//
+// Arithmetic contract.  Activations travel as f32 buffers; with bf16 weights the operands of the
+// matrix products (norm outputs, gated mixer outputs, feed-forward activations) are rounded to
+// bf16 values when they are stored, and keys / values are stored in the cache as bf16.  Norms,
+// angles, scores and weights, decays, the recurrent state and the residual sum are f32 always.
+// With f32 weights nothing is rounded.  Every output element is summed in an order that depends
+// only on its own position in its sequence (never on what else is in the batch or on how a prompt
+// was cut), so a token's result is the same bits in any batch.
+#include <math.h>
+
+#include <vector>
+
+#include "sd_common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld_f(const T* p);
+template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return (float)*p; }
+template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
+template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = (bf16_t)v; }
+
+__device__ __forceinline__ float maybe_round(float v, int round) { return round ? round_bf16(v) : v; }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+
+// Sum over a workgroup of up to 256 threads in a fixed order: butterfly inside each wave, then
+// the waves' sums in wave order.  `red` holds at least 4 floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int w = 1; w < n_waves; ++w) s += red[w];
+  return s;
+}
+
+// ------------------------------------------------------------------ rows in, rows out
+template <typename T>
+__global__ void embed_rows_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
+                                  float* __restrict__ x, int W, int vocab) {
+  const int r = blockIdx.x;
+  int tok = tokens[r];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) x[(size_t)r * W + c] = ld_f(table + (size_t)tok * W + c);
+}
+
+// out[i] = x[rows ? rows[i] : i] / sqrt(mean(x^2) + eps) * (offset + w)
+template <typename T>
+__global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                                    const T* __restrict__ w, float offset, float eps,
+                                    float* __restrict__ out, int W, int round) {
+  __shared__ float red[4];
+  const int i = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[i] : i) * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) ss = fmaf(xr[c], xr[c], ss);
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    out[(size_t)i * W + c] = maybe_round(xr[c] * rstd * (offset + ld_f(w + c)), round);
+}
+
+// Y[M, N] = X[M, K] W[N, K]^T + bias.  X is f32 (rounded to bf16 values on load when `round`;
+// with x2: the operand is relu(X) * X2, the gated feed-forward's activation).  Every output is
+// summed over k in ascending order, whatever the tile shape, so a row's bits do not depend on M.
+template <typename T, int BM, int BN, int TM, int TN>
+__global__ __launch_bounds__(256) void matmul_rows_kernel(
+    const float* __restrict__ X, const float* __restrict__ X2, int64_t ldx, const T* __restrict__ Wt,
+    const float* __restrict__ bias, float* __restrict__ Y, int64_t ldy, int M, int N, int K, int round) {
+  constexpr int BK = 16;
+  static_assert((BM / TM) * (BN / TN) == 256, "256 threads");
+  __shared__ float xs[BK][BM + 1];
+  __shared__ float ws[BK][BN + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid % (BN / TN), ty = tid / (BN / TN);
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  float acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int idx = tid; idx < BM * BK; idx += 256) {
+      const int m = idx / BK, kk = idx % BK;
+      float v = 0.f;
+      if (m0 + m < M && k0 + kk < K) {
+        v = X[(size_t)(m0 + m) * ldx + k0 + kk];
+        if (X2) v = fmaxf(v, 0.f) * X2[(size_t)(m0 + m) * ldx + k0 + kk];
+        v = maybe_round(v, round);
+      }
+      xs[kk][m] = v;
+    }
+    for (int idx = tid; idx < BN * BK; idx += 256) {
+      const int n = idx / BK, kk = idx % BK;
+      ws[kk][n] = (n0 + n < N && k0 + kk < K) ? ld_f(Wt + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = xs[kk][ty * TM + i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = ws[kk][tx * TN + j];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + ty * TM + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + tx * TN + j;
+      if (n < N) Y[(size_t)m * ldy + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ rotary embedding
+// One wave per (row, head).  Heads 0..Hq-1 are query heads at q, heads Hq..Hq+Hk-1 key heads at k.
+// The first `dims` channels are rotated in place: pair i is (i, i + dims/2) (layout 0) or
+// (2i, 2i + 1) (layout 1), by the angle pos * inv_freq[i], formed in f64 (the product of a position
+// in the thousands and an f32 frequency loses the low bits of the angle otherwise).  Then the
+// vector is divided by its root mean square (unit_norm) and multiplied by q_scale / k_scale.
+// Key heads with a cache: the finished key and the value row go to the paged cache.  Every lane
+// re-reads only what it wrote itself.
+template <typename T>
+__global__ void head_prep_kernel(float* __restrict__ q, float* __restrict__ k, const float* __restrict__ v,
+                                 int64_t ld, const int32_t* __restrict__ row_pos,
+                                 const int32_t* __restrict__ row_slot, int Hq, int Hk, int dk, int dv,
+                                 int dims, int layout, const double* __restrict__ inv_freq, int unit_norm,
+                                 float eps, float q_scale, float k_scale, T* __restrict__ k_cache,
+                                 T* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
+                                 int max_blocks, int page) {
+  const int r = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+  const bool is_q = hh < Hq;
+  const int head = is_q ? hh : hh - Hq;
+  float* vec = (is_q ? q : k) + (size_t)r * ld + (size_t)head * dk;
+  const int pos = row_pos[r];
+  float ss = 0.f;
+  for (int i = lane; i < dims / 2; i += 64) {
+    const double a = (double)pos * inv_freq[i];
+    const float cs = (float)cos(a), sn = (float)sin(a);
+    const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
+    const float u = vec[iu], w = vec[iv];
+    const float ru = u * cs - w * sn, rw = w * cs + u * sn;
+    vec[iu] = ru;
+    vec[iv] = rw;
+    ss = fmaf(ru, ru, ss);
+    ss = fmaf(rw, rw, ss);
+  }
+  for (int c = dims + lane; c < dk; c += 64) ss = fmaf(vec[c], vec[c], ss);
+  float scale = is_q ? q_scale : k_scale;
+  if (unit_norm) {
+    ss = wave_sum(ss);
+    scale *= 1.f / sqrtf(ss / (float)dk + eps);
+  }
+  T* kc = nullptr;
+  T* vc = nullptr;
+  if (!is_q && k_cache) {
+    const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+    const size_t at = ((size_t)pg * Hk + head) * page + pos % page;
+    kc = k_cache + at * dk;
+    vc = v_cache + at * dv;
+  }
+  for (int i = lane; i < dims / 2; i += 64) {
+    const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
+    const float ou = vec[iu] * scale, ov = vec[iv] * scale;
+    vec[iu] = ou;
+    vec[iv] = ov;
+    if (kc) {
+      st_f(kc + iu, ou);
+      st_f(kc + iv, ov);
+    }
+  }
+  for (int c = dims + lane; c < dk; c += 64) {
+    const float o = vec[c] * scale;
+    vec[c] = o;
+    if (kc) st_f(kc + c, o);
+  }
+  if (vc) {
+    const float* vr = v + (size_t)r * ld + (size_t)head * dv;
+    for (int c = lane; c < dv; c += 64) st_f(vc + c, vr[c]);
+  }
+}
+
+// decay[r, c] = sigmoid(z[r, c])^(1/tau) = exp(-softplus(-z) / tau)
+__global__ void sigmoid_power_kernel(const float* __restrict__ z, int64_t ldz, float inv_tau,
+                                     float* __restrict__ out, int n_cols) {
+  const int r = blockIdx.x;
+  for (int c = threadIdx.x; c < n_cols; c += blockDim.x) {
+    const float x = z[(size_t)r * ldz + c];
+    const float log_sig = x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
+    out[(size_t)r * n_cols + c] = expf(log_sig * inv_tau);
+  }
+}
+
+// ------------------------------------------------------------------ decayed outer-product scan
+// S <- diag(d_t) S + k_t v_t^T,  o_t = S^T q_t, token by token, per (entry, head).  A thread owns
+// 16 consecutive key channels of one value column; the strips' partial dot products are added in
+// strip order.  d_t: a factor per key channel (PER_CHANNEL, [rows, H*dk]) or per head ([H]).
+constexpr int kStrip = 16;
+template <bool PER_CHANNEL>
+__global__ __launch_bounds__(256) void decay_scan_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, int64_t ld,
+    const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ entries,
+    float* __restrict__ out, int H, int dk, int dv, int CT, int NS, int CH) {
+  extern __shared__ float lds[];
+  const int dkp = NS * kStrip;
+  float* qs = lds;                  // [CH][dkp]
+  float* ks = qs + CH * dkp;        // [CH][dkp]
+  float* ds = ks + CH * dkp;        // [CH][dkp] (PER_CHANNEL only)
+  float* vs = ds + (PER_CHANNEL ? CH * dkp : 0);  // [CH][CT]
+  float* part = vs + CH * CT;       // [CH][NS][CT]
+  const int tid = threadIdx.x, nthr = CT * NS;
+  const int c = tid % CT, s = tid / CT;
+  const int h = blockIdx.y, e = blockIdx.z;
+  const int col = blockIdx.x * CT + c;
+  const int slot = entries[4 * e], row0 = entries[4 * e + 1], len = entries[4 * e + 2],
+            pos0 = entries[4 * e + 3];
+  float* st = state + ((size_t)slot * H + h) * dk * dv;
+  const int r0 = s * kStrip;
+  float S[kStrip];
+#pragma unroll
+  for (int r = 0; r < kStrip; ++r)
+    S[r] = (pos0 > 0 && r0 + r < dk && col < dv) ? st[(size_t)(r0 + r) * dv + col] : 0.f;
+  const float dh = PER_CHANNEL ? 0.f : decay[h];
+  for (int t0 = 0; t0 < len; t0 += CH) {
+    const int nt = len - t0 < CH ? len - t0 : CH;
+    for (int idx = tid; idx < nt * dkp; idx += nthr) {
+      const int t = idx / dkp, ch = idx % dkp;
+      const size_t row = (size_t)(row0 + t0 + t);
+      const bool in = ch < dk;
+      qs[t * dkp + ch] = in ? q[row * ld + (size_t)h * dk + ch] : 0.f;
+      ks[t * dkp + ch] = in ? k[row * ld + (size_t)h * dk + ch] : 0.f;
+      if (PER_CHANNEL) ds[t * dkp + ch] = in ? decay[row * ((size_t)H * dk) + (size_t)h * dk + ch] : 0.f;
+    }
+    for (int idx = tid; idx < nt * CT; idx += nthr) {
+      const int t = idx / CT, cc = idx % CT;
+      const int vcol = blockIdx.x * CT + cc;
+      vs[t * CT + cc] = vcol < dv ? v[(size_t)(row0 + t0 + t) * ld + (size_t)h * dv + vcol] : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+      const float vv = vs[t * CT + c];
+      const float* qt = qs + t * dkp + r0;
+      const float* kt = ks + t * dkp + r0;
+      const float* dt = ds + t * dkp + r0;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < kStrip; ++r) {
+        const float d = PER_CHANNEL ? dt[r] : dh;
+        S[r] = fmaf(d, S[r], kt[r] * vv);
+        acc = fmaf(S[r], qt[r], acc);
+      }
+      part[(t * NS + s) * CT + c] = acc;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nt * CT; idx += nthr) {
+      const int t = idx / CT, cc = idx % CT;
+      const int ocol = blockIdx.x * CT + cc;
+      if (ocol >= dv) continue;
+      float o = part[(t * NS) * CT + cc];
+      for (int ss = 1; ss < NS; ++ss) o += part[(t * NS + ss) * CT + cc];
+      out[(size_t)(row0 + t0 + t) * ((size_t)H * dv) + (size_t)h * dv + ocol] = o;
+    }
+    __syncthreads();
+  }
+  if (col < dv) {
+#pragma unroll
+    for (int r = 0; r < kStrip; ++r)
+      if (r0 + r < dk) st[(size_t)(r0 + r) * dv + col] = S[r];
+  }
+}
+
+// y[r, h*dv + c] = o * (unit_norm ? rstd(o over the head) : 1) * (norm_w ? norm_w[c] : 1) * gate(g)
+// gate: 0 = silu, 1 = sigmoid.  One wave per (row, head).
+template <typename T>
+__global__ void head_post_kernel(const float* __restrict__ o, const float* __restrict__ g, int64_t ldg,
+                                 const T* __restrict__ norm_w, int unit_norm, float eps, int gate_kind,
+                                 float* __restrict__ y, int H, int dv, int round) {
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* orow = o + (size_t)r * H * dv + (size_t)h * dv;
+  const float* grow = g + (size_t)r * ldg + (size_t)h * dv;
+  float rstd = 1.f;
+  if (unit_norm) {
+    float ss = 0.f;
+    for (int c = lane; c < dv; c += 64) ss = fmaf(orow[c], orow[c], ss);
+    ss = wave_sum(ss);
+    rstd = 1.f / sqrtf(ss / (float)dv + eps);
+  }
+  for (int c = lane; c < dv; c += 64) {
+    const float gz = grow[c];
+    const float gate = gate_kind ? sigmoid_f(gz) : gz * sigmoid_f(gz);
+    float val = orow[c] * rstd;
+    if (norm_w) val *= ld_f(norm_w + c);
+    y[(size_t)r * H * dv + (size_t)h * dv + c] = maybe_round(val * gate, round);
+  }
+}
+
+// ------------------------------------------------------------------ window + pooled blocks
+// In-page slot of pooled block b, whose last token lies in logical page lp.
+__device__ __forceinline__ int pooled_slot(int b, int lp, int page, int pool) { return b - (lp * page) / pool; }
+
+// Mean key / value of every block of `pool` tokens that a new row completes, from the rows the
+// cache holds.  One wave per (row, kv head).
+template <typename T>
+__global__ void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                   float* __restrict__ pk_cache, float* __restrict__ pv_cache,
+                                   const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                                   const int32_t* __restrict__ block_tables, int max_blocks, int page,
+                                   int pslots, int G, int dk, int dv, int pool) {
+  const int r = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const int pos = row_pos[r];
+  if (pos % pool != pool - 1) return;
+  const int b = pos / pool;
+  const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
+  const int lp = pos / page;
+  const size_t dst = ((size_t)tbl[lp] * G + g) * pslots + pooled_slot(b, lp, page, pool);
+  for (int c = lane; c < dk + dv; c += 64) {
+    const bool is_k = c < dk;
+    const int cc = is_k ? c : c - dk;
+    const int d = is_k ? dk : dv;
+    const T* cache = is_k ? k_cache : v_cache;
+    float sum = 0.f;
+    for (int j = b * pool; j <= pos; ++j)
+      sum += ld_f(cache + (((size_t)tbl[j / page] * G + g) * page + j % page) * d + cc);
+    (is_k ? pk_cache : pv_cache)[dst * d + cc] = sum / (float)pool;
+  }
+}
+
+// Position i sees the tokens j with 0 <= i - j < window and the pooled blocks b with
+// b*pool + pool - 1 <= i - window.  Weight of a key: sigmoid(q.k * scale + head_bias[h]); the
+// weighted values are summed, not normalised.  One workgroup per (row, query head).
+constexpr int kAttnTile = 256;
+constexpr int kAttnCols = 4;  // value columns per lane: vdim <= 256
+template <typename T>
+__global__ __launch_bounds__(256) void window_pool_attn_kernel(
+    const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const float* __restrict__ pk_cache, const float* __restrict__ pv_cache,
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+    const int32_t* __restrict__ block_tables, int max_blocks, int page, int pslots, int H, int G, int dk,
+    int dv, int window, int pool, float scale, const float* __restrict__ head_bias,
+    float* __restrict__ out) {
+  extern __shared__ float lds[];
+  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [kAttnTile] cache row of the value
+  float* wt = reinterpret_cast<float*>(vat + kAttnTile);                 // [kAttnTile]
+  int* kind = reinterpret_cast<int*>(wt + kAttnTile);                    // [kAttnTile] 1 = pooled
+  float* qs = reinterpret_cast<float*>(kind + kAttnTile);                // [dk]
+  float* red = qs + dk;                                                  // [4][dv]
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int g = h / (H / G);
+  const int i = row_pos[r];
+  const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
+  for (int c = tid; c < dk; c += 256) qs[c] = q[(size_t)r * ldq + (size_t)h * dk + c];
+  const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
+  const int n_blocks = i - window + 1 >= 0 ? (i - window + 1) / pool : 0;
+  const int total = n_blocks + (i - t_first + 1);
+  const float bias = head_bias ? head_bias[h] : 0.f;
+  const int wave = tid >> 6, lane = tid & 63;
+  float acc[kAttnCols];
+#pragma unroll
+  for (int m = 0; m < kAttnCols; ++m) acc[m] = 0.f;
+  __syncthreads();
+  for (int base = 0; base < total; base += kAttnTile) {
+    const int idx = base + tid;
+    if (idx < total) {
+      float s = 0.f;
+      if (idx < n_blocks) {
+        const int last = idx * pool + pool - 1, lp = last / page;
+        const size_t at = ((size_t)tbl[lp] * G + g) * pslots + pooled_slot(idx, lp, page, pool);
+        const float* kr = pk_cache + at * dk;
+        for (int c = 0; c < dk; ++c) s = fmaf(qs[c], kr[c], s);
+        kind[tid] = 1;
+        vat[tid] = at;
+      } else {
+        const int j = t_first + (idx - n_blocks);
+        const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
+        const T* kr = k_cache + at * dk;
+        for (int c = 0; c < dk; ++c) s = fmaf(qs[c], ld_f(kr + c), s);
+        kind[tid] = 0;
+        vat[tid] = at;
+      }
+      wt[tid] = sigmoid_f(s * scale + bias);
+    }
+    __syncthreads();
+    const int n_here = total - base < kAttnTile ? total - base : kAttnTile;
+    for (int kk = wave; kk < n_here; kk += 4) {
+      const float w = wt[kk];
+      const size_t at = vat[kk];
+      if (kind[kk]) {
+        const float* vr = pv_cache + at * dv;
+#pragma unroll
+        for (int m = 0; m < kAttnCols; ++m)
+          if (lane + 64 * m < dv) acc[m] = fmaf(w, vr[lane + 64 * m], acc[m]);
+      } else {
+        const T* vr = v_cache + at * dv;
+#pragma unroll
+        for (int m = 0; m < kAttnCols; ++m)
+          if (lane + 64 * m < dv) acc[m] = fmaf(w, ld_f(vr + lane + 64 * m), acc[m]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int m = 0; m < kAttnCols; ++m)
+    if (lane + 64 * m < dv) red[wave * dv + lane + 64 * m] = acc[m];
+  __syncthreads();
+  for (int c = tid; c < dv; c += 256)
+    out[(size_t)r * H * dv + (size_t)h * dv + c] = ((red[c] + red[dv + c]) + red[2 * dv + c]) + red[3 * dv + c];
+}
+
+// x += sigmoid(z1) * a + sigmoid(z2) * b   (b == nullptr: one sublayer)
+__global__ void gated_residual_kernel(float* __restrict__ x, const float* __restrict__ z1,
+                                      const float* __restrict__ z2, int64_t ldz, const float* __restrict__ a,
+                                      const float* __restrict__ b, int W) {
+  const int r = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float add = sigmoid_f(z1[(size_t)r * ldz + c]) * a[(size_t)r * W + c];
+    if (b) add += sigmoid_f(z2[(size_t)r * ldz + c]) * b[(size_t)r * W + c];
+    x[(size_t)r * W + c] += add;
+  }
+}
+
+template <typename T>
+int launch_matmul(const float* X, const float* X2, int64_t ldx, const void* Wt, const float* bias, float* Y,
+                  int64_t ldy, int M, int N, int K, int round, hipStream_t st) {
+  if (M <= 16) {
+    dim3 grid((N + 127) / 128, (M + 15) / 16);
+    matmul_rows_kernel<T, 16, 128, 2, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round);
+  } else {
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    matmul_rows_kernel<T, 64, 64, 4, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round);
+  }
+  SD_CHECK_LAUNCH("sd_matmul_rows");
+  return SD_OK;
+}
+
+}  // namespace
+
+// ====================================================================== C entry points
+extern "C" int sd_matmul_rows(const float* x, const float* x2, int64_t ldx, const void* w, int w_f32,
+                              const float* bias, float* y, int64_t ldy, int M, int N, int K,
+                              sd_stream_t stream) {
+  SD_REQUIRE(x && w && y && M >= 1 && N >= 1 && K >= 1 && ldx >= K && ldy >= N, SD_ERR_INVALID,
+             "sd_matmul_rows: bad argument (M=%d N=%d K=%d)", M, N, K);
+  hipStream_t st = (hipStream_t)stream;
+  return w_f32 ? launch_matmul<float>(x, x2, ldx, w, bias, y, ldy, M, N, K, 0, st)
+               : launch_matmul<bf16_t>(x, x2, ldx, w, bias, y, ldy, M, N, K, 1, st);
+}
+
+extern "C" int sd_rmsnorm_rows(const float* x, const int32_t* rows, const void* w, int w_f32, float offset,
+                               float eps, float* out, int n, int W, sd_stream_t stream) {
+  SD_REQUIRE(x && w && out && n >= 1 && W >= 1, SD_ERR_INVALID, "sd_rmsnorm_rows: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32) rmsnorm_rows_kernel<float><<<n, 256, 0, st>>>(x, rows, (const float*)w, offset, eps, out, W, 0);
+  else rmsnorm_rows_kernel<bf16_t><<<n, 256, 0, st>>>(x, rows, (const bf16_t*)w, offset, eps, out, W, 1);
+  SD_CHECK_LAUNCH("sd_rmsnorm_rows");
+  return SD_OK;
+}
+
+extern "C" int sd_head_prep(float* q, float* k, const float* v, int64_t ld, const int32_t* row_pos,
+                            const int32_t* row_slot, int n_rows, int Hq, int Hk, int dk, int dv,
+                            int rot_dims, int rot_layout, const double* inv_freq, int unit_norm, float eps,
+                            float q_scale, float k_scale, void* k_cache, void* v_cache, int cache_f32,
+                            const int32_t* block_tables, int max_blocks, int page, sd_stream_t stream) {
+  SD_REQUIRE(q && k && row_pos && n_rows >= 1 && Hq >= 1 && Hk >= 1 && dk >= 1, SD_ERR_INVALID,
+             "sd_head_prep: bad argument");
+  SD_REQUIRE(rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq),
+             SD_ERR_INVALID, "sd_head_prep: rot_dims %d must be even, at most dim %d, with a frequency table",
+             rot_dims, dk);
+  SD_REQUIRE(!k_cache || (v_cache && v && row_slot && block_tables && page >= 1 && max_blocks >= 1),
+             SD_ERR_INVALID, "sd_head_prep: a cache needs values, slots and block tables");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, Hq + Hk);
+  if (cache_f32)
+    head_prep_kernel<float><<<grid, 64, 0, st>>>(q, k, v, ld, row_pos, row_slot, Hq, Hk, dk, dv, rot_dims,
+                                                 rot_layout, inv_freq, unit_norm, eps, q_scale, k_scale,
+                                                 (float*)k_cache, (float*)v_cache, block_tables, max_blocks, page);
+  else
+    head_prep_kernel<bf16_t><<<grid, 64, 0, st>>>(q, k, v, ld, row_pos, row_slot, Hq, Hk, dk, dv, rot_dims,
+                                                  rot_layout, inv_freq, unit_norm, eps, q_scale, k_scale,
+                                                  (bf16_t*)k_cache, (bf16_t*)v_cache, block_tables, max_blocks, page);
+  SD_CHECK_LAUNCH("sd_head_prep");
+  return SD_OK;
+}
+
+extern "C" int sd_sigmoid_power(const float* z, int64_t ldz, float tau, float* out, int n_rows, int n_cols,
+                                sd_stream_t stream) {
+  SD_REQUIRE(z && out && n_rows >= 1 && n_cols >= 1 && tau > 0.f, SD_ERR_INVALID, "sd_sigmoid_power: bad argument");
+  sigmoid_power_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(z, ldz, 1.f / tau, out, n_cols);
+  SD_CHECK_LAUNCH("sd_sigmoid_power");
+  return SD_OK;
+}
+
+extern "C" int sd_decay_scan(const float* q, const float* k, const float* v, int64_t ld, const float* decay,
+                             int per_channel, float* state, const int32_t* entries, int n_entries,
+                             float* out, int H, int dk, int dv, sd_stream_t stream) {
+  SD_REQUIRE(q && k && v && decay && state && entries && out && n_entries >= 1 && H >= 1 && dv >= 1,
+             SD_ERR_INVALID, "sd_decay_scan: bad argument");
+  SD_REQUIRE(dk >= 1 && dk <= 256, SD_ERR_UNSUPPORTED, "sd_decay_scan: key size %d outside 1..256", dk);
+  const int NS = (dk + kStrip - 1) / kStrip;
+  int CT = 256 / NS;
+  if (CT > dv) CT = dv;
+  if (CT > 64) CT = 64;
+  const int tiles = (dv + CT - 1) / CT;
+  const int CH = dk > 128 ? 8 : 16;
+  const int dkp = NS * kStrip;
+  const size_t lds = sizeof(float) * ((size_t)(per_channel ? 3 : 2) * CH * dkp + (size_t)CH * CT + (size_t)CH * NS * CT);
+  dim3 grid(tiles, H, n_entries);
+  hipStream_t st = (hipStream_t)stream;
+  if (per_channel)
+    decay_scan_kernel<true><<<grid, CT * NS, lds, st>>>(q, k, v, ld, decay, state, entries, out, H, dk, dv, CT, NS, CH);
+  else
+    decay_scan_kernel<false><<<grid, CT * NS, lds, st>>>(q, k, v, ld, decay, state, entries, out, H, dk, dv, CT, NS, CH);
+  SD_CHECK_LAUNCH("sd_decay_scan");
+  return SD_OK;
+}
+
+extern "C" int sd_head_post(const float* o, const float* g, int64_t ldg, const void* norm_w, int w_f32,
+                            int unit_norm, float eps, int gate_kind, float* y, int n_rows, int H, int dv,
+                            int round_bf16_out, sd_stream_t stream) {
+  SD_REQUIRE(o && g && y && n_rows >= 1 && H >= 1 && dv >= 1, SD_ERR_INVALID, "sd_head_post: bad argument");
+  dim3 grid(n_rows, H);
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32)
+    head_post_kernel<float><<<grid, 64, 0, st>>>(o, g, ldg, (const float*)norm_w, unit_norm, eps, gate_kind, y, H, dv, round_bf16_out);
+  else
+    head_post_kernel<bf16_t><<<grid, 64, 0, st>>>(o, g, ldg, (const bf16_t*)norm_w, unit_norm, eps, gate_kind, y, H, dv, round_bf16_out);
+  SD_CHECK_LAUNCH("sd_head_post");
+  return SD_OK;
+}
+
+extern "C" int sd_pooled_slots_per_page(int page, int pool) {
+  if (page < 1 || pool < 1) return 0;
+  return page / pool + 2;
+}
+
+extern "C" int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                        int cache_f32, float* pk_cache, float* pv_cache,
+                                        const int32_t* row_pos, const int32_t* row_slot,
+                                        const int32_t* block_tables, int max_blocks, int page, int n_rows,
+                                        int H, int G, int dk, int dv, int window, int pool, float scale,
+                                        const float* head_bias, float* out, sd_stream_t stream) {
+  SD_REQUIRE(q && k_cache && v_cache && pk_cache && pv_cache && row_pos && row_slot && block_tables && out,
+             SD_ERR_INVALID, "sd_window_pool_attention: null argument");
+  SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && pool >= 1 && page >= 1,
+             SD_ERR_INVALID, "sd_window_pool_attention: bad shape");
+  SD_REQUIRE(dv >= 1 && dv <= 64 * kAttnCols, SD_ERR_UNSUPPORTED,
+             "sd_window_pool_attention: value size %d outside 1..%d", dv, 64 * kAttnCols);
+  const int pslots = sd_pooled_slots_per_page(page, pool);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 gp(n_rows, G);
+  dim3 ga(n_rows, H);
+  const size_t lds = sizeof(float) * (size_t)(dk + kAttnTile * 2 + 4 * dv) + sizeof(unsigned long long) * kAttnTile + 16;
+  if (cache_f32) {
+    pool_blocks_kernel<float><<<gp, 64, 0, st>>>((const float*)k_cache, (const float*)v_cache, pk_cache, pv_cache,
+                                                 row_pos, row_slot, block_tables, max_blocks, page, pslots, G, dk, dv, pool);
+    SD_CHECK_LAUNCH("sd_window_pool_attention (pool)");
+    window_pool_attn_kernel<float><<<ga, 256, lds, st>>>(q, ldq, (const float*)k_cache, (const float*)v_cache, pk_cache,
+                                                         pv_cache, row_pos, row_slot, block_tables, max_blocks, page,
+                                                         pslots, H, G, dk, dv, window, pool, scale, head_bias, out);
+  } else {
+    pool_blocks_kernel<bf16_t><<<gp, 64, 0, st>>>((const bf16_t*)k_cache, (const bf16_t*)v_cache, pk_cache, pv_cache,
+                                                  row_pos, row_slot, block_tables, max_blocks, page, pslots, G, dk, dv, pool);
+    SD_CHECK_LAUNCH("sd_window_pool_attention (pool)");
+    window_pool_attn_kernel<bf16_t><<<ga, 256, lds, st>>>(q, ldq, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pk_cache,
+                                                          pv_cache, row_pos, row_slot, block_tables, max_blocks, page,
+                                                          pslots, H, G, dk, dv, window, pool, scale, head_bias, out);
+  }
+  SD_CHECK_LAUNCH("sd_window_pool_attention");
+  return SD_OK;
+}
+
+extern "C" int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* a,
+                                 const float* b, int n_rows, int W, sd_stream_t stream) {
+  SD_REQUIRE(x && z1 && a && (!b || z2) && n_rows >= 1 && W >= 1, SD_ERR_INVALID, "sd_gated_residual: bad argument");
+  gated_residual_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(x, z1, z2, ldz, a, b, W);
+  SD_CHECK_LAUNCH("sd_gated_residual");
+  return SD_OK;
+}
+
+// ====================================================================== the layer-list model
+struct sd_seq_model {
+  sd_seq_model_desc d;
+  std::vector<sd_seq_layer> layers;
+};
+
+namespace {
+struct InCols {  // column offsets inside a layer's fused input projection
+  int q, k, v, g, r1, r2, gate, up, a1, total;
+};
+InCols in_cols(const sd_seq_layer& l, int W) {
+  InCols c;
+  int at = 0;
+  c.q = at;    at += l.heads * l.dim;
+  c.k = at;    at += l.kv_heads * l.dim;
+  c.v = at;    at += l.kv_heads * l.vdim;
+  c.g = at;    at += l.heads * l.vdim;
+  c.r1 = at;   at += W;
+  c.r2 = at;   at += l.ff > 0 ? W : 0;
+  c.gate = at; at += l.ff;
+  c.up = at;   at += l.ff;
+  c.a1 = at;   at += l.kind == SD_MIX_CHANNEL_DECAY ? l.rank : 0;
+  c.total = at;
+  return c;
+}
+inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
+struct SeqWs {
+  size_t x, h, proj, dec, o, y, mix, ffo, hout, total;
+};
+SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
+  const int W = m.d.width;
+  size_t proj = 0, hk = 0, hv = 0;
+  for (const sd_seq_layer& l : m.layers) {
+    const size_t t = in_cols(l, W).total;
+    proj = t > proj ? t : proj;
+    const size_t a = (size_t)l.heads * l.dim, b = (size_t)l.heads * l.vdim;
+    hk = a > hk ? a : hk;
+    hv = b > hv ? b : hv;
+  }
+  SeqWs w;
+  size_t off = 0;
+  const size_t R = (size_t)rows, f = sizeof(float);
+  w.x = off;    off += al(R * W * f);
+  w.h = off;    off += al(R * W * f);
+  w.proj = off; off += al(R * proj * f);
+  w.dec = off;  off += al(R * hk * f);   // low-rank decay logits, then decays
+  w.o = off;    off += al(R * hv * f);
+  w.y = off;    off += al(R * hv * f);
+  w.mix = off;  off += al(R * W * f);
+  w.ffo = off;  off += al(R * W * f);
+  w.hout = off; off += al((size_t)(n_out > 0 ? n_out : 1) * W * f);
+  w.total = off;
+  return w;
+}
+}  // namespace
+
+extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
+  if (!desc || !desc->layers || desc->n_layers < 1 || desc->width < 1 || desc->vocab < 1 || !desc->embed ||
+      !desc->final_norm_w) {
+    sd_set_error("sd_seq_model_create: null descriptor, no layers or a missing table");
+    return nullptr;
+  }
+  sd_seq_model* m = new sd_seq_model;
+  m->d = *desc;
+  m->layers.assign(desc->layers, desc->layers + desc->n_layers);
+  m->d.layers = m->layers.data();
+  for (int i = 0; i < desc->n_layers; ++i) {
+    const sd_seq_layer& l = m->layers[i];
+    const char* bad = nullptr;
+    if (l.kind != SD_MIX_HEAD_DECAY && l.kind != SD_MIX_CHANNEL_DECAY && l.kind != SD_MIX_WINDOW_POOL) bad = "unknown mixer";
+    else if (l.heads < 1 || l.kv_heads < 1 || l.heads % l.kv_heads || l.dim < 1 || l.vdim < 1) bad = "head counts / sizes";
+    else if (!l.norm_w || !l.w_in || !l.b_in || !l.w_o || (l.ff > 0 && !l.w_down) || l.ff < 0) bad = "a null weight";
+    else if (l.rot_dims < 0 || l.rot_dims > l.dim || l.rot_dims % 2 || (l.rot_dims && !l.inv_freq)) bad = "rotary dims";
+    else if (l.kind == SD_MIX_WINDOW_POOL) {
+      if (!l.k_cache || !l.v_cache || !l.pk_cache || !l.pv_cache || l.window < 1 || l.pool < 1 || l.vdim > 256)
+        bad = "window attention needs caches, window >= 1, pool >= 1, vdim <= 256";
+    } else {
+      if (l.heads != l.kv_heads || !l.state || l.dim > 256) bad = "a recurrent mixer needs a state, dim <= 256, no grouped heads";
+      else if (l.kind == SD_MIX_HEAD_DECAY && !l.head_decay) bad = "decay per head missing";
+      else if (l.kind == SD_MIX_CHANNEL_DECAY && (!l.w_a2 || !l.b_a2 || l.rank < 1 || !(l.tau > 0.f))) bad = "channel decay needs its low-rank pair and tau > 0";
+    }
+    if (bad) {
+      sd_set_error("sd_seq_model_create: layer %d: %s", i, bad);
+      delete m;
+      return nullptr;
+    }
+  }
+  return m;
+}
+
+extern "C" void sd_seq_model_destroy(sd_seq_model* m) { delete m; }
+
+extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out) {
+  if (!m || max_rows < 1) return 0;
+  return plan_seq(*m, max_rows, max_out).total;
+}
+
+#define SQ_TRY(expr)                \
+  do {                              \
+    int rc__ = (expr);              \
+    if (rc__ != SD_OK) return rc__; \
+  } while (0)
+
+extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void* workspace,
+                                    size_t workspace_bytes, sd_stream_t stream) {
+  SD_REQUIRE(m && b && workspace, SD_ERR_INVALID, "sd_seq_model_forward: null argument");
+  SD_REQUIRE(b->n_rows >= 1 && b->n_entries >= 1 && b->tokens && b->row_pos && b->row_slot && b->entries,
+             SD_ERR_INVALID, "sd_seq_model_forward: empty batch or null array");
+  SD_REQUIRE(b->n_out >= 0 && (b->n_out == 0 || (b->out_rows && b->logits)), SD_ERR_INVALID,
+             "sd_seq_model_forward: wanted rows need out_rows and logits");
+  const SeqWs w = plan_seq(*m, b->n_rows, b->n_out);
+  SD_REQUIRE(workspace_bytes >= w.total, SD_ERR_WORKSPACE, "sd_seq_model_forward: workspace %zu < %zu bytes",
+             workspace_bytes, w.total);
+  SD_REQUIRE(sd_aligned16(workspace), SD_ERR_INVALID, "sd_seq_model_forward: workspace unaligned");
+  const sd_seq_model_desc& d = m->d;
+  const int W = d.width, R = b->n_rows, f32 = d.weights_f32, rnd = !f32;
+  hipStream_t st = (hipStream_t)stream;
+  char* base = (char*)workspace;
+  float* x = (float*)(base + w.x);
+  float* h = (float*)(base + w.h);
+  float* proj = (float*)(base + w.proj);
+  float* dec = (float*)(base + w.dec);
+  float* o = (float*)(base + w.o);
+  float* y = (float*)(base + w.y);
+  float* mix = (float*)(base + w.mix);
+  float* ffo = (float*)(base + w.ffo);
+  float* hout = (float*)(base + w.hout);
+
+  if (f32) embed_rows_kernel<float><<<R, 256, 0, st>>>(b->tokens, (const float*)d.embed, x, W, d.vocab);
+  else embed_rows_kernel<bf16_t><<<R, 256, 0, st>>>(b->tokens, (const bf16_t*)d.embed, x, W, d.vocab);
+  SD_CHECK_LAUNCH("sd_seq_model_forward (embed)");
+
+  for (int li = 0; li < d.n_layers; ++li) {
+    const sd_seq_layer& l = m->layers[li];
+    const InCols c = in_cols(l, W);
+    const int64_t ld = c.total;
+    const int H = l.heads, G = l.kv_heads, dk = l.dim, dv = l.vdim;
+    SQ_TRY(sd_rmsnorm_rows(x, nullptr, l.norm_w, f32, 1.f, d.norm_eps, h, R, W, stream));
+    // every matrix that reads h, in one product: q k v g | residual gates | ff gate, up | low-rank decay
+    SQ_TRY(sd_matmul_rows(h, nullptr, W, l.w_in, f32, l.b_in, proj, ld, R, c.total, W, stream));
+    if (l.kind == SD_MIX_WINDOW_POOL) {
+      SQ_TRY(sd_head_prep(proj + c.q, proj + c.k, proj + c.v, ld, b->row_pos, b->row_slot, R, H, G, dk, dv,
+                          l.rot_dims, l.rot_layout, l.inv_freq, l.qk_unit_norm, d.norm_eps, l.q_scale, l.k_scale,
+                          l.k_cache, l.v_cache, f32, b->block_tables, b->max_blocks, b->page, stream));
+      SQ_TRY(sd_window_pool_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, l.pk_cache, l.pv_cache,
+                                      b->row_pos, b->row_slot, b->block_tables, b->max_blocks, b->page, R, H, G,
+                                      dk, dv, l.window, l.pool, l.score_scale, l.head_bias, o, stream));
+      SQ_TRY(sd_head_post(o, proj + c.g, ld, nullptr, f32, 0, d.norm_eps, 1, y, R, H, dv, rnd, stream));
+    } else {
+      SQ_TRY(sd_head_prep(proj + c.q, proj + c.k, nullptr, ld, b->row_pos, b->row_slot, R, H, H, dk, dv,
+                          l.rot_dims, l.rot_layout, l.inv_freq, l.qk_unit_norm, d.norm_eps, l.q_scale, l.k_scale,
+                          nullptr, nullptr, f32, nullptr, 0, 0, stream));
+      const bool pc = l.kind == SD_MIX_CHANNEL_DECAY;
+      if (pc) {
+        // decay logits through the low-rank pair (its first half came out of the fused product)
+        float* z = o;  // free until the scan writes it; the scan reads `dec`
+        SQ_TRY(sd_matmul_rows(proj + c.a1, nullptr, ld, l.w_a2, f32, l.b_a2, z, (int64_t)H * dk, R, H * dk, l.rank, stream));
+        SQ_TRY(sd_sigmoid_power(z, (int64_t)H * dk, l.tau, dec, R, H * dk, stream));
+      }
+      SQ_TRY(sd_decay_scan(proj + c.q, proj + c.k, proj + c.v, ld, pc ? dec : l.head_decay, pc, l.state,
+                           b->entries, b->n_entries, o, H, dk, dv, stream));
+      SQ_TRY(sd_head_post(o, proj + c.g, ld, l.head_norm_w, f32, 1, d.norm_eps, 0, y, R, H, dv, rnd, stream));
+    }
+    SQ_TRY(sd_matmul_rows(y, nullptr, (int64_t)H * dv, l.w_o, f32, nullptr, mix, W, R, W, H * dv, stream));
+    if (l.ff > 0)
+      SQ_TRY(sd_matmul_rows(proj + c.gate, proj + c.up, ld, l.w_down, f32, nullptr, ffo, W, R, W, l.ff, stream));
+    SQ_TRY(sd_gated_residual(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, mix, l.ff > 0 ? ffo : nullptr,
+                             R, W, stream));
+    if (b->layer_out) {
+      const hipError_t e = hipMemcpyAsync(b->layer_out + (size_t)li * R * W, x, (size_t)R * W * sizeof(float),
+                                          hipMemcpyDeviceToDevice, st);
+      SD_REQUIRE(e == hipSuccess, SD_ERR_HIP, "sd_seq_model_forward: copying a layer's output: %s",
+                 hipGetErrorString(e));
+    }
+  }
+  if (b->n_out > 0) {
+    SQ_TRY(sd_rmsnorm_rows(x, b->out_rows, d.final_norm_w, f32, 1.f, d.norm_eps, hout, b->n_out, W, stream));
+    SQ_TRY(sd_matmul_rows(hout, nullptr, W, d.embed, f32, nullptr, b->logits, d.vocab, b->n_out, d.vocab, W, stream));
+  }
+  return SD_OK;
+}

@@ -108,3 +108,100 @@ class PagedKVCache:
 
     def nbytes(self) -> int:
         return 2 * self.k.numel() * 2
+
+
+# ---------------------------------------------------------------------------------------------
+# Caches of layer-list models (config.SeqModelConfig): per-sequence recurrent states in slots, and
+# pages of plain key / value rows (plus pooled rows) for windowed attention layers.
+class OutOfSlots(RuntimeError):
+    pass
+
+
+class SlotAllocator:
+    """Sequence slots: the row of a block table, and of every recurrent layer's state tensor."""
+
+    def __init__(self, n: int):
+        self.n = n
+        self._free = list(range(n - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise OutOfSlots("every sequence slot is taken")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        if slot in self._free:
+            raise ValueError(f"slot {slot} is free already")
+        self._free.append(slot)
+
+
+class SeqCache:
+    """What the sequences of a layer-list model keep on the device.
+
+    Recurrent layers: state[layer] f32 [slots, heads, dim, vdim]; a slot's state needs no clearing
+    when the slot is taken again (a sequence that starts at position 0 starts from zero).
+    Window layers: k / v [pages, kv_heads, PAGE, dim | vdim] in the serving dtype and the pooled
+    means pk / pv f32 [pages, kv_heads, pooled slots per page, dim | vdim]; one page table per
+    slot serves all window layers."""
+
+    def __init__(self, cfg, dtype: torch.dtype, max_seqs: int, num_pages: int, max_seq_len: int,
+                 device="cuda"):
+        from . import ops
+        self.cfg, self.dtype = cfg, dtype
+        self.page = PAGE
+        self.slots = SlotAllocator(max_seqs)
+        self.allocator = PageAllocator(num_pages)
+        self.max_blocks_per_seq = max(1, (max_seq_len + PAGE - 1) // PAGE)
+        self.block_tables = torch.zeros(max_seqs, self.max_blocks_per_seq, dtype=torch.int32, device=device)
+        self._host_tables: List[List[int]] = [[] for _ in range(max_seqs)]
+        self.state: Dict[int, torch.Tensor] = {}
+        self.k: Dict[int, torch.Tensor] = {}
+        self.v: Dict[int, torch.Tensor] = {}
+        self.pk: Dict[int, torch.Tensor] = {}
+        self.pv: Dict[int, torch.Tensor] = {}
+        self.has_pages = False
+        for i, l in enumerate(cfg.layers):
+            m = l.mixer
+            if m.kind == "attention":
+                self.has_pages = True
+                ps = ops.pooled_slots_per_page(PAGE, m.pool)
+                self.k[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.dim, dtype=dtype, device=device)
+                self.v[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.vdim, dtype=dtype, device=device)
+                self.pk[i] = torch.zeros(num_pages, m.kv_heads, ps, m.dim, dtype=torch.float32, device=device)
+                self.pv[i] = torch.zeros(num_pages, m.kv_heads, ps, m.vdim, dtype=torch.float32, device=device)
+            else:
+                self.state[i] = torch.zeros(max_seqs, m.heads, m.dim, m.vdim, dtype=torch.float32, device=device)
+
+    def pages_of(self, slot: int) -> List[int]:
+        return self._host_tables[slot]
+
+    def ensure_capacity(self, slot: int, n_tokens: int) -> None:
+        """Slot `slot` owns pages for positions 0..n_tokens-1 afterwards (window layers only)."""
+        if not self.has_pages:
+            return
+        need = (n_tokens + PAGE - 1) // PAGE
+        if need > self.max_blocks_per_seq:
+            raise OutOfPages(f"sequence of {n_tokens} tokens exceeds max_seq_len")
+        tbl = self._host_tables[slot]
+        if len(tbl) >= need:
+            return
+        if need - len(tbl) > self.allocator.num_free:
+            raise OutOfPages("KV cache is out of pages")
+        first_new = len(tbl)
+        while len(tbl) < need:
+            tbl.append(self.allocator.alloc())
+        self.block_tables[slot, first_new:need].copy_(torch.tensor(tbl[first_new:], dtype=torch.int32),
+                                                      non_blocking=False)
+
+    def release(self, slot: int) -> None:
+        self.allocator.free(self._host_tables[slot])
+        self._host_tables[slot] = []
+        self.slots.free(slot)
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for d in (self.state, self.k, self.v, self.pk, self.pv)
+                   for t in d.values())

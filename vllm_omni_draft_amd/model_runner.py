@@ -198,3 +198,96 @@ class DecoderModel:
                                           ws.data_ptr(), ws.numel(),
                                           ops._stream())
         _lib.check(rc, "sd_model_forward")
+
+
+# ---------------------------------------------------------------------------------------------
+_MIX_KIND = {"retention": 0, "gla": 1, "attention": 2}
+
+
+class SeqModel:
+    """Host handle of a layer-list model (config.SeqModelConfig) on one GPU: the native descriptor
+    over the weights and the caches (sd_seq_model_create), and a workspace that grows with the
+    largest batch seen.  forward() enqueues one pass over a ragged batch; nothing here computes."""
+
+    def __init__(self, weights, cache):
+        from .weights import SeqModelWeights
+        if not isinstance(weights, SeqModelWeights):
+            raise TypeError("SeqModel needs SeqModelWeights")
+        if cache.dtype != weights.dtype:
+            raise ValueError("the cache must hold the serving dtype")
+        self.weights, self.cache = weights, cache
+        self.cfg = weights.cfg
+        cfg = self.cfg
+        f32 = weights.dtype == torch.float32
+        layers = (_lib.SeqLayer * cfg.n_layers)()
+        for i, (spec, t) in enumerate(zip(cfg.layers, weights.layers)):
+            m = spec.mixer
+            rec = m.kind != "attention"
+            layers[i] = _lib.SeqLayer(
+                kind=_MIX_KIND[m.kind], heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
+                ff=spec.ff, rot_dims=m.rot_dims, rot_layout=int(m.rot_layout == "interleaved"),
+                inv_freq=_ptr(t.inv_freq), qk_unit_norm=int(m.kind == "attention"),
+                q_scale=m.dim ** -0.5 if m.kind == "gla" else 1.0,
+                k_scale=m.dim ** -0.5 if m.kind == "retention" else 1.0,
+                score_scale=m.scale, window=m.window, pool=m.pool, rank=m.rank, tau=m.tau,
+                norm_w=_ptr(t.norm_w), w_in=_ptr(t.w_in), b_in=_ptr(t.b_in), w_o=_ptr(t.w_o),
+                w_down=_ptr(t.w_down), w_a2=_ptr(t.w_a2), b_a2=_ptr(t.b_a2),
+                head_decay=_ptr(t.head_decay), head_bias=_ptr(t.head_bias),
+                head_norm_w=_ptr(t.head_norm_w),
+                state=_ptr(cache.state.get(i)) if rec else None,
+                k_cache=_ptr(cache.k.get(i)), v_cache=_ptr(cache.v.get(i)),
+                pk_cache=_ptr(cache.pk.get(i)), pv_cache=_ptr(cache.pv.get(i)))
+        desc = _lib.SeqModelDesc(n_layers=cfg.n_layers, width=cfg.width, vocab=cfg.vocab,
+                                 weights_f32=int(f32), norm_eps=cfg.norm_eps, embed=_ptr(weights.embed),
+                                 final_norm_w=_ptr(weights.final_norm_w), layers=layers)
+        self._handle = _lib.load().sd_seq_model_create(C.byref(desc))
+        if not self._handle:
+            raise _lib.SdError(f"sd_seq_model_create failed: {_lib.last_error()}")
+        self.workspace = None
+        self._ws_rows = self._ws_out = 0
+
+    def __del__(self):
+        h = getattr(self, "_handle", None)
+        if h:
+            try:
+                _lib.load().sd_seq_model_destroy(h)
+            except Exception:
+                pass
+            self._handle = None
+
+    def _ensure_workspace(self, rows: int, n_out: int) -> None:
+        if self.workspace is not None and rows <= self._ws_rows and n_out <= self._ws_out:
+            return
+        self._ws_rows, self._ws_out = max(rows, self._ws_rows), max(n_out, self._ws_out, 1)
+        n = _lib.load().sd_seq_model_workspace_bytes(self._handle, self._ws_rows, self._ws_out)
+        self.workspace = torch.empty(int(n), dtype=torch.uint8, device=self.weights.embed.device)
+
+    def forward(self, n_rows: int, n_entries: int, tokens, row_pos, row_slot, entries, n_out: int,
+                out_rows, logits, layer_out=None) -> None:
+        """int32 device tensors tokens / row_pos / row_slot [n_rows], entries [n_entries, 4]
+        {slot, first row, rows, first position}, out_rows [n_out]; logits f32 [n_out, vocab];
+        layer_out (optional) f32 [n_layers, n_rows, width] receives the residual after each layer."""
+        for t, name in ((tokens, "tokens"), (row_pos, "row_pos"), (row_slot, "row_slot"), (entries, "entries")):
+            if t.dtype != torch.int32 or not t.is_contiguous() or not t.is_cuda:
+                raise _lib.SdError(f"{name} must be a contiguous int32 device tensor")
+        if tokens.numel() < n_rows or row_pos.numel() < n_rows or row_slot.numel() < n_rows \
+                or entries.numel() < 4 * n_entries:
+            raise _lib.SdError("batch arrays shorter than the batch")
+        if n_out and (out_rows is None or out_rows.dtype != torch.int32 or out_rows.numel() < n_out
+                      or logits is None or logits.dtype != torch.float32 or not logits.is_contiguous()
+                      or logits.numel() < n_out * self.cfg.vocab):
+            raise _lib.SdError("wanted rows need int32 out_rows and contiguous float32 logits [n_out, vocab]")
+        if layer_out is not None and (layer_out.dtype != torch.float32 or not layer_out.is_contiguous()
+                                      or layer_out.numel() < self.cfg.n_layers * n_rows * self.cfg.width):
+            raise _lib.SdError("layer_out must be contiguous float32 [n_layers, n_rows, width]")
+        self._ensure_workspace(n_rows, n_out)
+        c = self.cache
+        batch = _lib.SeqBatch(n_rows=n_rows, n_entries=n_entries, tokens=tokens.data_ptr(),
+                              row_pos=row_pos.data_ptr(), row_slot=row_slot.data_ptr(),
+                              entries=entries.data_ptr(), block_tables=c.block_tables.data_ptr(),
+                              max_blocks=c.max_blocks_per_seq, page=c.page, n_out=n_out,
+                              out_rows=_ptr(out_rows) if n_out else None,
+                              logits=_ptr(logits) if n_out else None, layer_out=_ptr(layer_out))
+        rc = _lib.load().sd_seq_model_forward(self._handle, C.byref(batch), self.workspace.data_ptr(),
+                                              self.workspace.numel(), ops._stream())
+        _lib.check(rc, "sd_seq_model_forward")

@@ -1030,3 +1030,12 @@ def chain_down_qkv(state, down_w: TiledWeight, act, h, norm_w, eps, qkv_w: Tiled
         _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(seq_lens), pos_offset,
         B, q_len, Hq, Hkv, D, _stream()), "sd_chain_down_qkv")
     return q
+
+
+# ---------------------------------------------------------------- layer-list models
+def pooled_slots_per_page(page: int, pool: int) -> int:
+    """Pooled entries per cache page of a window layer with blocks of `pool` tokens."""
+    n = int(_lib.load().sd_pooled_slots_per_page(int(page), int(pool)))
+    if n < 1:
+        raise _lib.SdError(f"pooled_slots_per_page: bad page {page} / pool {pool}")
+    return n

@@ -313,3 +313,153 @@ def from_safetensors_dir(cfg: ModelConfig, model_dir: str, device="cuda",
     if cfg.arch == "opt" and "decoder.embed_tokens.weight" in state:
         state = {"model." + k if k.startswith("decoder.") else k: v for k, v in state.items()}
     return from_state_dict(cfg, state, device, fp8=fp8, head_subset=head_subset)
+
+
+# ---------------------------------------------------------------------------------------------
+# Layer-list models (config.SeqModelConfig): row-major matrices in the dtype the model is served
+# in (bfloat16 or float32), every matrix of a layer that reads the normed input stacked into one.
+@dataclass
+class SeqLayerTensors:
+    norm_w: torch.Tensor
+    w_in: torch.Tensor            # [q | k | v | g | r1 | r2 | ff gate | ff up | a1] x width
+    b_in: torch.Tensor            # f32 bias of w_in (the residual gates' biases; zero elsewhere)
+    w_o: torch.Tensor
+    w_down: Optional[torch.Tensor] = None
+    w_a2: Optional[torch.Tensor] = None
+    b_a2: Optional[torch.Tensor] = None       # f32
+    head_decay: Optional[torch.Tensor] = None  # f32 [heads]
+    head_bias: Optional[torch.Tensor] = None   # f32 [heads]
+    head_norm_w: Optional[torch.Tensor] = None
+    inv_freq: Optional[torch.Tensor] = None    # f64 [rot_dims / 2]
+
+
+@dataclass
+class SeqModelWeights:
+    cfg: "SeqModelConfig"
+    dtype: torch.dtype
+    embed: torch.Tensor
+    final_norm_w: torch.Tensor
+    layers: List[SeqLayerTensors]
+
+    def tensors(self):
+        yield self.embed
+        yield self.final_norm_w
+        for l in self.layers:
+            for t in vars(l).values():
+                if t is not None:
+                    yield t
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.tensors())
+
+
+def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
+                        dtype: torch.dtype = torch.bfloat16) -> SeqModelWeights:
+    """Tensors under the checkpoint's names ('embed', 'final.norm', 'l<i>.norm1', 'l<i>.mix.*',
+    'l<i>.mlp.*', 'l<i>.rg1', 'l<i>.rg1.b', ...) -> device tensors in the serving dtype."""
+    if dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("a layer-list model is served in bfloat16 or float32")
+    W = cfg.width
+
+    def get(name, shape):
+        if name not in state:
+            raise KeyError(f"checkpoint has no tensor {name!r}")
+        t = state[name]
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    def dev(t, dt=None):
+        return t.to(dt or dtype).contiguous().to(device)
+
+    layers = []
+    for i, l in enumerate(cfg.layers):
+        m, p = l.mixer, f"l{i}."
+        H, G, dk, dv = m.heads, m.kv_heads, m.dim, m.vdim
+        parts = [get(p + "mix.q", (H * dk, W)), get(p + "mix.k", (G * dk, W)), get(p + "mix.v", (G * dv, W)),
+                 get(p + "mix.g", (H * dv, W)), get(p + "rg1", (W, W))]
+        bias = [torch.zeros(H * dk + G * dk + G * dv + H * dv), get(p + "rg1.b", (W,)).float()]
+        if l.ff:
+            parts += [get(p + "rg2", (W, W)), get(p + "mlp.gate", (l.ff, W)), get(p + "mlp.up", (l.ff, W))]
+            bias += [get(p + "rg2.b", (W,)).float(), torch.zeros(2 * l.ff)]
+        if m.kind == "gla":
+            parts.append(get(p + "mix.a1", (m.rank, W)))
+            bias.append(torch.zeros(m.rank))
+        lt = SeqLayerTensors(
+            norm_w=dev(get(p + "norm1", (W,))), w_in=dev(torch.cat([t.float() for t in parts])),
+            b_in=dev(torch.cat(bias), torch.float32), w_o=dev(get(p + "mix.o", (W, H * dv))))
+        if l.ff:
+            lt.w_down = dev(get(p + "mlp.down", (W, l.ff)))
+        if m.kind == "gla":
+            lt.w_a2 = dev(get(p + "mix.a2", (H * dk, m.rank)))
+            lt.b_a2 = dev(get(p + "mix.a2.b", (H * dk,)), torch.float32)
+            lt.head_norm_w = dev(get(p + "mix.norm", (dv,)))
+        if m.kind == "retention":
+            lt.head_decay = dev(torch.tensor(m.decay, dtype=torch.float64), torch.float32)
+        if m.kind == "attention":
+            lt.head_bias = dev(get(p + "mix.pb", (H,)), torch.float32)
+        if m.rot_dims:
+            i2 = torch.arange(m.rot_dims // 2, dtype=torch.float64)
+            lt.inv_freq = dev(torch.tensor(m.rot_base, dtype=torch.float64) ** (-2.0 * i2 / m.rot_dims),
+                              torch.float64)
+        layers.append(lt)
+    return SeqModelWeights(cfg, dtype, dev(get("embed", (cfg.vocab, W))), dev(get("final.norm", (W,))), layers)
+
+
+def seq_from_safetensors_dir(cfg, model_dir: str, device="cuda",
+                             dtype: torch.dtype = torch.bfloat16) -> SeqModelWeights:
+    from safetensors import safe_open
+
+    files = sorted(glob.glob(os.path.join(model_dir, "*.safetensors")))
+    if not files:
+        raise FileNotFoundError(f"no *.safetensors under {model_dir}")
+    state: Dict[str, torch.Tensor] = {}
+    for fn in files:
+        with safe_open(fn, framework="pt", device="cpu") as f:
+            for key in f.keys():
+                state[key] = f.get_tensor(key)
+    return seq_from_state_dict(cfg, state, device, dtype)
+
+
+def seq_random_state(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """Seeded random tensors under the checkpoint's names (bfloat16 values), scaled so that
+    activations stay of order one: for benchmarks and examples."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg.width
+
+    def rn(*shape, s):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    st = {"embed": rn(cfg.vocab, W, s=1.0), "final.norm": rn(W, s=0.1)}
+    for i, l in enumerate(cfg.layers):
+        m, p = l.mixer, f"l{i}."
+        H, G, dk, dv = m.heads, m.kv_heads, m.dim, m.vdim
+        st[p + "norm1"] = rn(W, s=0.1)
+        for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv), ("g", H * dv)):
+            st[p + "mix." + nm] = rn(rows, W, s=W ** -0.5)
+        st[p + "mix.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
+        if m.kind == "attention":
+            st[p + "mix.pb"] = rn(H, s=1.0) - 4.0
+        if m.kind == "gla":
+            st[p + "mix.norm"] = 1 + rn(dv, s=0.1)
+            st[p + "mix.a1"] = rn(m.rank, W, s=W ** -0.5)
+            st[p + "mix.a2"] = rn(H * dk, m.rank, s=m.rank ** -0.5)
+            st[p + "mix.a2.b"] = rn(H * dk, s=1.0) + 3.0
+        st[p + "rg1"], st[p + "rg1.b"] = rn(W, W, s=W ** -0.5), rn(W, s=0.5)
+        if l.ff:
+            st[p + "mlp.gate"], st[p + "mlp.up"] = rn(l.ff, W, s=W ** -0.5), rn(l.ff, W, s=W ** -0.5)
+            st[p + "mlp.down"] = rn(W, l.ff, s=l.ff ** -0.5)
+            st[p + "rg2"], st[p + "rg2.b"] = rn(W, W, s=W ** -0.5), rn(W, s=0.5)
+    return st
+
+
+def load_model(model_dir: str, device="cuda", dtype: torch.dtype = torch.bfloat16, **kw):
+    """Configuration and weights of a checkpoint folder, whatever model class its config.json
+    names: (SeqModelConfig, SeqModelWeights) or (ModelConfig, ModelWeights)."""
+    from .config import SeqModelConfig, load_model_config
+    cfg = load_model_config(model_dir)
+    if isinstance(cfg, SeqModelConfig):
+        return cfg, seq_from_safetensors_dir(cfg, model_dir, device, dtype)
+    if dtype != torch.bfloat16:
+        raise ValueError("Hugging Face decoders are served in bfloat16 (or fp8 weights) only")
+    return cfg, from_safetensors_dir(cfg, model_dir, device, **kw)
