@@ -1039,3 +1039,113 @@ def pooled_slots_per_page(page: int, pool: int) -> int:
     if n < 1:
         raise _lib.SdError(f"pooled_slots_per_page: bad page {page} / pool {pool}")
     return n
+
+
+def _f32(t: torch.Tensor, name: str) -> None:
+    _need(t, torch.float32, name)
+
+
+def _wkind(w: torch.Tensor, name: str) -> int:
+    if w.dtype not in (torch.float32, torch.bfloat16) or not w.is_contiguous():
+        raise _lib.SdError(f"{name}: a contiguous float32 or bfloat16 tensor")
+    return int(w.dtype == torch.float32)
+
+
+def matmul_rows(x: torch.Tensor, w: torch.Tensor, bias=None, x2=None) -> torch.Tensor:
+    """x [M, K] f32 times w [N, K] (f32, or bf16: x is then rounded to bf16 values) -> f32 [M, N];
+    x2: the operand is relu(x) * x2."""
+    _f32(x, "x")
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K or (x2 is not None and x2.shape != x.shape):
+        raise _lib.SdError("matmul_rows: shapes do not fit")
+    y = torch.empty(M, N, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().sd_matmul_rows(_p(x), _p(x2), K, _p(w), _wkind(w, "w"), _p(bias), _p(y), N, M, N, K,
+                                          _stream()), "sd_matmul_rows")
+    return y
+
+
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, offset: float = 0.0, rows=None) -> torch.Tensor:
+    _f32(x, "x")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty(n, x.shape[1], dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().sd_rmsnorm_rows(_p(x), _p(rows), _p(w), _wkind(w, "w"), float(offset), float(eps),
+                                           _p(out), n, x.shape[1], _stream()), "sd_rmsnorm_rows")
+    return out
+
+
+def head_prep(q, k, row_pos, Hq, Hk, dk, *, rot_dims=0, rot_layout=0, inv_freq=None, unit_norm=False,
+              eps=1e-5, q_scale=1.0, k_scale=1.0, v=None, dv=0, k_cache=None, v_cache=None, row_slot=None,
+              block_tables=None) -> None:
+    """In place on q [rows, Hq*dk] and k [rows, Hk*dk] (each contiguous); see sd_head_prep."""
+    _f32(q, "q")
+    _f32(k, "k")
+    n = q.shape[0]
+    # the entry point takes one row stride: q, k (and v) as columns of one buffer
+    buf = torch.cat([q, k] + ([v] if v is not None else []), dim=1).contiguous()
+    ld = buf.shape[1]
+    qp, kp = buf.data_ptr(), buf.data_ptr() + 4 * q.shape[1]
+    vp = kp + 4 * k.shape[1] if v is not None else None
+    _lib.check(_lib.load().sd_head_prep(
+        qp, kp, vp, ld, _p(row_pos), _p(row_slot), n, Hq, Hk, dk, dv, rot_dims, rot_layout, _p(inv_freq),
+        int(unit_norm), float(eps), float(q_scale), float(k_scale), _p(k_cache), _p(v_cache),
+        int(k_cache is not None and k_cache.dtype == torch.float32), _p(block_tables),
+        block_tables.shape[1] if block_tables is not None else 0, PAGE, _stream()), "sd_head_prep")
+    q.copy_(buf[:, :q.shape[1]])
+    k.copy_(buf[:, q.shape[1]:q.shape[1] + k.shape[1]])
+
+
+def sigmoid_power(z: torch.Tensor, tau: float) -> torch.Tensor:
+    _f32(z, "z")
+    out = torch.empty_like(z)
+    _lib.check(_lib.load().sd_sigmoid_power(_p(z), z.shape[1], float(tau), _p(out), z.shape[0], z.shape[1],
+                                            _stream()), "sd_sigmoid_power")
+    return out
+
+
+def decay_scan(q, k, v, decay, state, entries, H, dk, dv) -> torch.Tensor:
+    """q, k [rows, H*dk], v [rows, H*dv] f32; decay [H] or [rows, H*dk]; state [slots, H, dk, dv]
+    (updated); entries int32 [n, 4] {slot, first row, rows, first position}."""
+    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (decay, "decay"), (state, "state")):
+        _f32(t, nm)
+    _need(entries, torch.int32, "entries")
+    n = q.shape[0]
+    buf = torch.cat([q, k, v], dim=1).contiguous()
+    ld = buf.shape[1]
+    out = torch.empty(n, H * dv, dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().sd_decay_scan(buf.data_ptr(), buf.data_ptr() + 4 * H * dk, buf.data_ptr() + 8 * H * dk,
+                                         ld, _p(decay), int(decay.dim() == 2), _p(state), _p(entries),
+                                         entries.shape[0], _p(out), H, dk, dv, _stream()), "sd_decay_scan")
+    return out
+
+
+def head_post(o, g, H, dv, *, norm_w=None, unit_norm=False, eps=1e-5, gate="silu", round_bf16=False):
+    _f32(o, "o")
+    _f32(g, "g")
+    y = torch.empty_like(o)
+    _lib.check(_lib.load().sd_head_post(_p(o), _p(g), g.shape[1], _p(norm_w),
+                                        _wkind(norm_w, "norm_w") if norm_w is not None else 1, int(unit_norm),
+                                        float(eps), {"silu": 0, "sigmoid": 1}[gate], _p(y), o.shape[0], H, dv,
+                                        int(round_bf16), _stream()), "sd_head_post")
+    return y
+
+
+def window_pool_attention(q, k_cache, v_cache, pk_cache, pv_cache, row_pos, row_slot, block_tables, H, G,
+                          dk, dv, window, pool, scale, head_bias=None) -> torch.Tensor:
+    """q f32 [rows, H*dk] (prepared); caches as kv_cache.SeqCache lays them out; returns f32
+    [rows, H*dv].  Also fills the pooled entries of blocks that these rows complete."""
+    _f32(q, "q")
+    out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().sd_window_pool_attention(
+        _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(pk_cache),
+        _p(pv_cache), _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0],
+        H, G, dk, dv, window, pool, float(scale), _p(head_bias), _p(out), _stream()), "sd_window_pool_attention")
+    return out
+
+
+def gated_residual(x, z1, a, z2=None, b=None) -> None:
+    """x += sigmoid(z1) * a (+ sigmoid(z2) * b), in place; all f32 [rows, W]."""
+    for t, nm in ((x, "x"), (z1, "z1"), (a, "a")):
+        _f32(t, nm)
+    _lib.check(_lib.load().sd_gated_residual(_p(x), _p(z1), _p(z2), x.shape[1], _p(a), _p(b), x.shape[0],
+                                             x.shape[1], _stream()), "sd_gated_residual")
