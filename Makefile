@@ -31,11 +31,11 @@ $(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/sd_common.h include/sd_amd.h
 $(LIB): $(OBJS)
 	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(OBJS) -L/opt/rocm/lib -lrccl -Wl,-rpath,/opt/rocm/lib
 
-# The part of the library that layer-list models (sequence mixers, sampling) need, for a first
+# The part of the library that layer-list models (sequence mixers, linear layers, sampling) need, for a first
 # run in a fresh checkout that should not wait for every kernel family to compile.  The package
 # loads it only where the whole library has not been built.
 SEQ_LIB  := vllm_omni_draft_amd/libsd_seq.so
-SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_sampling.o
+SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_sampling.o $(CSRC)/sd_linear.o $(CSRC)/sd_linear_wide.o
 $(SEQ_LIB): $(SEQ_OBJS)
 	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(SEQ_OBJS)
 seq: $(SEQ_LIB)

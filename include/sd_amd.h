@@ -1043,9 +1043,9 @@ int sd_matmul_rows(const float* x, const float* x2, int64_t ldx, const void* w, 
                    const float* bias, float* y, int64_t ldy, int M, int N, int K,
                    sd_stream_t stream);
 /* out[i] = x[rows ? rows[i] : i] / sqrt(mean(x^2) + eps) * (offset + w): offset 1 for a weight
- * stored around zero, 0 for a plain weight.                                                */
+ * stored around zero, 0 for a plain weight.  out_bf16 (or NULL): the same rows as bf16.       */
 int sd_rmsnorm_rows(const float* x, const int32_t* rows, const void* w, int w_f32, float offset,
-                    float eps, float* out, int n, int W, sd_stream_t stream);
+                    float eps, float* out, void* out_bf16, int n, int W, sd_stream_t stream);
 /* Per (row, head), in place on q [rows, Hq*dk] and k [rows, Hk*dk] (row stride ld): rotary
  * embedding of the first rot_dims channels (rot_layout 0: channel i pairs with i + rot_dims/2;
  * 1: channel 2i with 2i+1; angle row_pos * inv_freq[i], inv_freq f64 [rot_dims/2]), then a
@@ -1069,10 +1069,11 @@ int sd_decay_scan(const float* q, const float* k, const float* v, int64_t ld, co
                   int per_channel, float* state, const int32_t* entries, int n_entries,
                   float* out, int H, int dk, int dv, sd_stream_t stream);
 /* y = o * (unit_norm ? 1/rms(o over the head) : 1) * (norm_w ? norm_w[c] : 1) * gate(g);
- * gate_kind 0: g*sigmoid(g), 1: sigmoid(g).  o, y [rows, H*dv]; g row stride ldg.            */
+ * gate_kind 0: g*sigmoid(g), 1: sigmoid(g).  o, y [rows, H*dv]; g row stride ldg; y_bf16 (or
+ * NULL): the same as bf16.                                                                 */
 int sd_head_post(const float* o, const float* g, int64_t ldg, const void* norm_w, int w_f32,
-                 int unit_norm, float eps, int gate_kind, float* y, int n_rows, int H, int dv,
-                 int round_bf16_out, sd_stream_t stream);
+                 int unit_norm, float eps, int gate_kind, float* y, void* y_bf16, int n_rows, int H,
+                 int dv, int round_bf16_out, sd_stream_t stream);
 /* Pooled entries a page of the pooled caches holds (blocks of `pool` tokens ending in it). */
 int sd_pooled_slots_per_page(int page, int pool);
 /* Sliding-window attention with pooled blocks and sigmoid weights over the cache sd_head_prep
@@ -1087,9 +1088,15 @@ int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, c
                              const int32_t* block_tables, int max_blocks, int page, int n_rows,
                              int H, int G, int dk, int dv, int window, int pool, float scale,
                              const float* head_bias, float* out, sd_stream_t stream);
-/* x += sigmoid(z1) * a + sigmoid(z2) * b (b, z2 may be NULL); x, a, b [rows, W].            */
-int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* a,
-                      const float* b, int n_rows, int W, sd_stream_t stream);
+/* x += sigmoid(z1 + c1) * a + sigmoid(z2 + c2) * b (b, z2 and the bias rows c1, c2 [W] may be
+ * NULL); x, a, b [rows, W].                                                                */
+int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
+                      const float* c2, const float* a, const float* b, int n_rows, int W,
+                      sd_stream_t stream);
+/* out_bf16[r, c] = relu(gate[r, c]) * up[r, c]: a gated feed-forward's activation as the bf16
+ * operand of sd_linear / sd_linear_wide.                                                   */
+int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, void* out_bf16, int n_rows,
+                     int F, sd_stream_t stream);
 
 typedef enum {
   SD_MIX_HEAD_DECAY = 0,    /* recurrence with a fixed decay per head (retention) */
@@ -1100,7 +1107,10 @@ typedef enum {
 /* One layer: h = norm(x); x += sigmoid(r1) * mixer(h) + sigmoid(r2) * ff(h).  w_in stacks every
  * matrix that reads h, rows in this order: q [heads*dim], k [kv_heads*dim], v [kv_heads*vdim],
  * g [heads*vdim], r1 [width], r2 [width] and the feed-forward's gate [ff], up [ff] (if ff > 0),
- * a1 [rank] (channel decay); b_in is its f32 bias.                                         */
+ * a1 [rank] (channel decay).  A matrix is given row-major (w_in, w_o, w_down; the model's
+ * element type) or, bf16 only and with an input width that is a multiple of 32, as
+ * SD_TILE_PLAIN tiles (sd_tile_weights): it then runs through sd_linear (up to 16 rows) and
+ * sd_linear_wide, the kernels of the other decoders.                                       */
 typedef struct {
   int kind;
   int heads, kv_heads, dim, vdim;
@@ -1114,9 +1124,13 @@ typedef struct {
   float tau;
   const void* norm_w;      /* [width], stored around zero */
   const void* w_in;
-  const float* b_in;
+  const void* w_in_tiled;
+  const float* r1_bias;    /* [width] f32 bias of the mixer's residual gate, or NULL */
+  const float* r2_bias;    /* the feed-forward's */
   const void* w_o;         /* [width, heads*vdim] */
+  const void* w_o_tiled;
   const void* w_down;      /* [width, ff] or NULL */
+  const void* w_down_tiled;
   const void* w_a2;        /* [heads*dim, rank] or NULL */
   const float* b_a2;
   const float* head_decay; /* [heads] or NULL */
@@ -1134,6 +1148,7 @@ typedef struct {
   int weights_f32;         /* element type of every weight and of the k / v caches */
   float norm_eps;
   const void* embed;       /* [vocab, width]; also the output head */
+  const void* head_tiled;  /* NULL, or the same table as SD_TILE_PLAIN tiles for the head */
   const void* final_norm_w;
   const sd_seq_layer* layers; /* copied */
 } sd_seq_model_desc;

@@ -63,18 +63,22 @@ SHAPES = {
                        layer("retention", heads=1, dim=40, vdim=72, rot_dims=2, decay=[0.875], ff=24),
                        layer("attention", heads=4, kv_heads=4, dim=16, vdim=8, window=20, pool=32, ff=24)],
                       width=40, vocab=50),
+    # widths that are multiples of 32: bfloat16 serving takes the tiled linear kernels everywhere
+    "aligned": model_cfg([layer("gla", heads=4, dim=32, vdim=16, rank=32, ff=160),
+                          layer("attention", heads=4, kv_heads=2, dim=32, vdim=24, window=12, pool=2, ff=64),
+                          layer("retention", heads=2, dim=16, vdim=48, ff=0)], width=128, vocab=176),
     "wide_heads": model_cfg([layer("gla", heads=2, dim=136, vdim=80, rank=5),
                              layer("attention", heads=2, kv_heads=1, dim=72, vdim=136, window=33, pool=3)],
                             width=48, vocab=64),
 }
 
 
-def build(cfg, dtype=torch.float32, seed=0, **eng_kw):
+def build(cfg, dtype=torch.float32, seed=0, tiled=True, **eng_kw):
     from vllm_omni_draft_amd import config, weights
     from vllm_omni_draft_amd.seq_engine import SeqEngine, SeqEngineConfig
     st = P.random_model(cfg, seed)
     mc = config.puguzen_config(cfg, {k: tuple(v.shape) for k, v in st.items()})
-    w = weights.seq_from_state_dict(mc, st, DEV, dtype)
+    w = weights.seq_from_state_dict(mc, st, DEV, dtype, tiled=tiled)
     kw = dict(max_seqs=4, max_tokens=1024)
     kw.update(eng_kw)
     return st, SeqEngine(w, SeqEngineConfig(**kw))
@@ -115,8 +119,9 @@ def test_rmsnorm_rows(W):
     out = ops.rmsnorm_rows(dev(x), dev(w), 1e-5, offset=1.0)
     assert rel(out, P.offset_rms_norm(x.double(), w.double(), 1e-5)) < 1e-6
     rows = i32([4, 0])
-    out = ops.rmsnorm_rows(dev(x), dev(w), 1e-3, offset=0.0, rows=rows)
+    out, out_b = ops.rmsnorm_rows(dev(x), dev(w), 1e-3, offset=0.0, rows=rows, bf16_copy=True)
     assert rel(out, P.unit_rms(x.double()[[4, 0]], 1e-3) * w.double()) < 1e-6
+    assert torch.equal(out_b, out.to(torch.bfloat16))
 
 
 @pytest.mark.parametrize("layout,dk,dims", [(0, 16, 16), (0, 24, 12), (1, 24, 8), (1, 70, 70), (1, 8, 0)])
@@ -204,6 +209,12 @@ def test_gated_residual():
     xd = dev(x)
     ops.gated_residual(xd, dev(z1), dev(a))
     assert rel(xd, x + torch.sigmoid(z1) * a) < 1e-6
+    c1, c2 = torch.randn(50, generator=g), torch.randn(50, generator=g)
+    xd = dev(x)
+    ops.gated_residual(xd, dev(z1), dev(a), dev(z2), dev(b), dev(c1), dev(c2))
+    assert rel(xd, x + torch.sigmoid(z1 + c1) * a + torch.sigmoid(z2 + c2) * b) < 1e-6
+    act = ops.relu_mul_rows(dev(z1), dev(z2))
+    assert torch.equal(act.cpu(), (torch.relu(z1) * z2).to(torch.bfloat16))
 
 
 class _AttnBed:
@@ -312,22 +323,33 @@ def test_prompt_logits_match_the_plain_model(shape):
 
 
 @pytest.mark.parametrize("shape", sorted(SHAPES))
-def test_bfloat16_serving_stays_close(shape):
+@pytest.mark.parametrize("tiled", [False, True])
+def test_bfloat16_serving_stays_close(shape, tiled):
     cfg = SHAPES[shape]
-    st, eng = build(cfg, torch.bfloat16)
+    st, eng = build(cfg, torch.bfloat16, tiled=tiled)
     toks = prompt(cfg, 60)
     logits = eng.step([("a", toks, list(range(60)))])
     assert rel(logits, oracle_logits(cfg, st, toks)) < 0.03
+    # 300 rows: more than one call of the many-row linear kernels
+    toks = prompt(cfg, 300, 4)
+    logits = eng.step([("b", toks, list(range(280, 300)))])
+    assert rel(logits, oracle_logits(cfg, st, toks)[280:]) < 0.03
 
 
 @pytest.mark.parametrize("shape", sorted(SHAPES))
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_cut_anywhere_batched_anyhow(shape, dtype):
+@pytest.mark.parametrize("mode", ["float32", "bfloat16-plain", "bfloat16-tiled"])
+def test_cut_anywhere_batched_anyhow(shape, mode):
     """The same three prompts: each alone and whole; token by token; in portions down to two
-    tokens; all three in mixed batches.  Logits agree to rounding (in fact to the bit: every sum
-    is taken in an order fixed by the token's own position)."""
+    tokens; all three in mixed batches.  Logits agree to rounding.  With the plain kernels they
+    agree to the bit (every sum is taken in an order fixed by the token's own position); the tiled
+    linear kernels have one summation order for up to 16 rows and another above."""
     cfg = SHAPES[shape]
-    st, eng = build(cfg, dtype)
+    dtype = torch.float32 if mode == "float32" else torch.bfloat16
+    st, eng = build(cfg, dtype, tiled=mode.endswith("tiled"))
+
+    def same(a, b):
+        return rel(a, b) < 1e-2 if mode.endswith("tiled") else torch.equal(a, b)
+
     lens = [71, 19, 40]
     toks = [prompt(cfg, n, i) for i, n in enumerate(lens)]
     whole = []
@@ -340,7 +362,7 @@ def test_cut_anywhere_batched_anyhow(shape, dtype):
     # token by token
     rows = [eng.step([("d", [t], [0])]).cpu() for t in toks[1]]
     eng.finish("d")
-    assert torch.equal(torch.cat(rows), whole[1])
+    assert same(torch.cat(rows), whole[1])
     # portions of changing size
     cuts, at, got = [2, 17, 2, 3, 31, 1, 2, 13], 0, []
     for c in cuts:
@@ -351,7 +373,7 @@ def test_cut_anywhere_batched_anyhow(shape, dtype):
         at += c
     assert at == lens[0]
     eng.finish("p")
-    assert torch.equal(torch.cat(got), whole[0])
+    assert same(torch.cat(got), whole[0])
     # mixed batches: portions of some beside single tokens of others, requests joining and leaving
     at = [0, 0, 0]
     got = [[], [], []]
@@ -370,7 +392,7 @@ def test_cut_anywhere_batched_anyhow(shape, dtype):
             at[i] += len(e[1])
     assert at == lens
     for i in range(3):
-        assert torch.equal(torch.cat(got[i]), whole[i]), i
+        assert same(torch.cat(got[i]), whole[i]), i
 
 
 def test_slots_and_pages_are_used_again():
@@ -474,7 +496,7 @@ def test_sampling_through_the_worker_is_seeded_per_request():
     cfg = SHAPES["three_kinds"]
     st = P.random_model(cfg, 3)
     mc = config.puguzen_config(cfg, {k: tuple(v.shape) for k, v in st.items()})
-    w = weights.seq_from_state_dict(mc, st, DEV, torch.bfloat16)
+    w = weights.seq_from_state_dict(mc, st, DEV, torch.float32)   # (bit-equal rows in any batch)
 
     def run(batch_mates):
         worker = SeqWorker(SeqWorkerConfig(w, max_num_seqs=4, max_model_len=64))

@@ -81,14 +81,16 @@ class SeqLayer(C.Structure):
                 ("rot_dims", i32), ("rot_layout", i32), ("inv_freq", vp), ("qk_unit_norm", i32),
                 ("q_scale", C.c_float), ("k_scale", C.c_float), ("score_scale", C.c_float),
                 ("window", i32), ("pool", i32), ("rank", i32), ("tau", C.c_float),
-                ("norm_w", vp), ("w_in", vp), ("b_in", vp), ("w_o", vp), ("w_down", vp), ("w_a2", vp),
+                ("norm_w", vp), ("w_in", vp), ("w_in_tiled", vp), ("r1_bias", vp), ("r2_bias", vp), ("w_o", vp),
+                ("w_o_tiled", vp), ("w_down", vp), ("w_down_tiled", vp), ("w_a2", vp),
                 ("b_a2", vp), ("head_decay", vp), ("head_bias", vp), ("head_norm_w", vp), ("state", vp),
                 ("k_cache", vp), ("v_cache", vp), ("pk_cache", vp), ("pv_cache", vp)]
 
 
 class SeqModelDesc(C.Structure):
     _fields_ = [("n_layers", i32), ("width", i32), ("vocab", i32), ("weights_f32", i32),
-                ("norm_eps", C.c_float), ("embed", vp), ("final_norm_w", vp), ("layers", C.POINTER(SeqLayer))]
+                ("norm_eps", C.c_float), ("embed", vp), ("head_tiled", vp), ("final_norm_w", vp),
+                ("layers", C.POINTER(SeqLayer))]
 
 
 class SeqBatch(C.Structure):
@@ -209,16 +211,17 @@ SIGNATURES = {
     "sd_graph_end": (i32, [vp, C.POINTER(vp)]),
     "sd_graph_launch": (i32, [vp, vp]),
     "sd_matmul_rows": (i32, [vp, vp, i64, vp, i32, vp, vp, i64, i32, i32, i32, vp]),
-    "sd_rmsnorm_rows": (i32, [vp, vp, vp, i32, C.c_float, C.c_float, vp, i32, i32, vp]),
+    "sd_rmsnorm_rows": (i32, [vp, vp, vp, i32, C.c_float, C.c_float, vp, vp, i32, i32, vp]),
     "sd_head_prep": (i32, [vp, vp, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, i32, C.c_float,
                            C.c_float, C.c_float, vp, vp, i32, vp, i32, i32, vp]),
     "sd_sigmoid_power": (i32, [vp, i64, C.c_float, vp, i32, i32, vp]),
     "sd_decay_scan": (i32, [vp, vp, vp, i64, vp, i32, vp, vp, i32, vp, i32, i32, i32, vp]),
-    "sd_head_post": (i32, [vp, vp, i64, vp, i32, i32, C.c_float, i32, vp, i32, i32, i32, i32, vp]),
+    "sd_head_post": (i32, [vp, vp, i64, vp, i32, i32, C.c_float, i32, vp, vp, i32, i32, i32, i32, vp]),
     "sd_pooled_slots_per_page": (i32, [i32, i32]),
     "sd_window_pool_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                        i32, i32, i32, C.c_float, vp, vp, vp]),
-    "sd_gated_residual": (i32, [vp, vp, vp, i64, vp, vp, i32, i32, vp]),
+    "sd_gated_residual": (i32, [vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, vp]),
+    "sd_relu_mul_rows": (i32, [vp, vp, i64, vp, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),
     "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32]),

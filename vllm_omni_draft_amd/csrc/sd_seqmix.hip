@@ -51,11 +51,11 @@ __global__ void embed_rows_kernel(const int32_t* __restrict__ tokens, const T* _
   for (int c = threadIdx.x; c < W; c += blockDim.x) x[(size_t)r * W + c] = ld_f(table + (size_t)tok * W + c);
 }
 
-// out[i] = x[rows ? rows[i] : i] / sqrt(mean(x^2) + eps) * (offset + w)
+// out[i] = x[rows ? rows[i] : i] / sqrt(mean(x^2) + eps) * (offset + w); out_b: the same as bf16
 template <typename T>
 __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
                                     const T* __restrict__ w, float offset, float eps,
-                                    float* __restrict__ out, int W, int round) {
+                                    float* __restrict__ out, bf16_t* __restrict__ out_b, int W, int round) {
   __shared__ float red[4];
   const int i = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[i] : i) * W;
@@ -63,8 +63,11 @@ __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* 
   for (int c = threadIdx.x; c < W; c += blockDim.x) ss = fmaf(xr[c], xr[c], ss);
   ss = block_sum(ss, red);
   const float rstd = 1.f / sqrtf(ss / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += blockDim.x)
-    out[(size_t)i * W + c] = maybe_round(xr[c] * rstd * (offset + ld_f(w + c)), round);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = maybe_round(xr[c] * rstd * (offset + ld_f(w + c)), round);
+    out[(size_t)i * W + c] = v;
+    if (out_b) out_b[(size_t)i * W + c] = (bf16_t)v;
+  }
 }
 
 // Y[M, N] = X[M, K] W[N, K]^T + bias.  X is f32 (rounded to bf16 values on load when `round`;
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
 template <typename T>
 __global__ void head_post_kernel(const float* __restrict__ o, const float* __restrict__ g, int64_t ldg,
                                  const T* __restrict__ norm_w, int unit_norm, float eps, int gate_kind,
-                                 float* __restrict__ y, int H, int dv, int round) {
+                                 float* __restrict__ y, bf16_t* __restrict__ y_b, int H, int dv, int round) {
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + (size_t)r * H * dv + (size_t)h * dv;
   const float* grow = g + (size_t)r * ldg + (size_t)h * dv;
@@ -306,7 +309,9 @@ __global__ void head_post_kernel(const float* __restrict__ o, const float* __res
     const float gate = gate_kind ? sigmoid_f(gz) : gz * sigmoid_f(gz);
     float val = orow[c] * rstd;
     if (norm_w) val *= ld_f(norm_w + c);
-    y[(size_t)r * H * dv + (size_t)h * dv + c] = maybe_round(val * gate, round);
+    const float res = maybe_round(val * gate, round);
+    y[(size_t)r * H * dv + (size_t)h * dv + c] = res;
+    if (y_b) y_b[(size_t)r * H * dv + (size_t)h * dv + c] = (bf16_t)res;
   }
 }
 
@@ -422,16 +427,26 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(
     out[(size_t)r * H * dv + (size_t)h * dv + c] = ((red[c] + red[dv + c]) + red[2 * dv + c]) + red[3 * dv + c];
 }
 
-// x += sigmoid(z1) * a + sigmoid(z2) * b   (b == nullptr: one sublayer)
+// x += sigmoid(z1 + c1) * a + sigmoid(z2 + c2) * b   (b == nullptr: one sublayer; c1, c2 may be null)
 __global__ void gated_residual_kernel(float* __restrict__ x, const float* __restrict__ z1,
-                                      const float* __restrict__ z2, int64_t ldz, const float* __restrict__ a,
+                                      const float* __restrict__ z2, int64_t ldz, const float* __restrict__ c1,
+                                      const float* __restrict__ c2, const float* __restrict__ a,
                                       const float* __restrict__ b, int W) {
   const int r = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float add = sigmoid_f(z1[(size_t)r * ldz + c]) * a[(size_t)r * W + c];
-    if (b) add += sigmoid_f(z2[(size_t)r * ldz + c]) * b[(size_t)r * W + c];
+    float add = sigmoid_f(z1[(size_t)r * ldz + c] + (c1 ? c1[c] : 0.f)) * a[(size_t)r * W + c];
+    if (b) add += sigmoid_f(z2[(size_t)r * ldz + c] + (c2 ? c2[c] : 0.f)) * b[(size_t)r * W + c];
     x[(size_t)r * W + c] += add;
   }
+}
+
+// out[r, c] = bf16(relu(gate[r, c]) * up[r, c]): the gated feed-forward's activation as the bf16
+// operand of the tiled linear kernels
+__global__ void relu_mul_rows_kernel(const float* __restrict__ gate, const float* __restrict__ up, int64_t ld,
+                                     bf16_t* __restrict__ out, int F) {
+  const int r = blockIdx.x;
+  for (int c = threadIdx.x; c < F; c += blockDim.x)
+    out[(size_t)r * F + c] = (bf16_t)(fmaxf(gate[(size_t)r * ld + c], 0.f) * up[(size_t)r * ld + c]);
 }
 
 template <typename T>
@@ -462,11 +477,12 @@ extern "C" int sd_matmul_rows(const float* x, const float* x2, int64_t ldx, cons
 }
 
 extern "C" int sd_rmsnorm_rows(const float* x, const int32_t* rows, const void* w, int w_f32, float offset,
-                               float eps, float* out, int n, int W, sd_stream_t stream) {
+                               float eps, float* out, void* out_bf16, int n, int W, sd_stream_t stream) {
   SD_REQUIRE(x && w && out && n >= 1 && W >= 1, SD_ERR_INVALID, "sd_rmsnorm_rows: bad argument");
   hipStream_t st = (hipStream_t)stream;
-  if (w_f32) rmsnorm_rows_kernel<float><<<n, 256, 0, st>>>(x, rows, (const float*)w, offset, eps, out, W, 0);
-  else rmsnorm_rows_kernel<bf16_t><<<n, 256, 0, st>>>(x, rows, (const bf16_t*)w, offset, eps, out, W, 1);
+  bf16_t* ob = (bf16_t*)out_bf16;
+  if (w_f32) rmsnorm_rows_kernel<float><<<n, 256, 0, st>>>(x, rows, (const float*)w, offset, eps, out, ob, W, 0);
+  else rmsnorm_rows_kernel<bf16_t><<<n, 256, 0, st>>>(x, rows, (const bf16_t*)w, offset, eps, out, ob, W, 1);
   SD_CHECK_LAUNCH("sd_rmsnorm_rows");
   return SD_OK;
 }
@@ -530,15 +546,15 @@ extern "C" int sd_decay_scan(const float* q, const float* k, const float* v, int
 }
 
 extern "C" int sd_head_post(const float* o, const float* g, int64_t ldg, const void* norm_w, int w_f32,
-                            int unit_norm, float eps, int gate_kind, float* y, int n_rows, int H, int dv,
-                            int round_bf16_out, sd_stream_t stream) {
+                            int unit_norm, float eps, int gate_kind, float* y, void* y_bf16, int n_rows, int H,
+                            int dv, int round_bf16_out, sd_stream_t stream) {
   SD_REQUIRE(o && g && y && n_rows >= 1 && H >= 1 && dv >= 1, SD_ERR_INVALID, "sd_head_post: bad argument");
   dim3 grid(n_rows, H);
   hipStream_t st = (hipStream_t)stream;
   if (w_f32)
-    head_post_kernel<float><<<grid, 64, 0, st>>>(o, g, ldg, (const float*)norm_w, unit_norm, eps, gate_kind, y, H, dv, round_bf16_out);
+    head_post_kernel<float><<<grid, 64, 0, st>>>(o, g, ldg, (const float*)norm_w, unit_norm, eps, gate_kind, y, (bf16_t*)y_bf16, H, dv, round_bf16_out);
   else
-    head_post_kernel<bf16_t><<<grid, 64, 0, st>>>(o, g, ldg, (const bf16_t*)norm_w, unit_norm, eps, gate_kind, y, H, dv, round_bf16_out);
+    head_post_kernel<bf16_t><<<grid, 64, 0, st>>>(o, g, ldg, (const bf16_t*)norm_w, unit_norm, eps, gate_kind, y, (bf16_t*)y_bf16, H, dv, round_bf16_out);
   SD_CHECK_LAUNCH("sd_head_post");
   return SD_OK;
 }
@@ -584,11 +600,21 @@ extern "C" int sd_window_pool_attention(const float* q, int64_t ldq, const void*
   return SD_OK;
 }
 
-extern "C" int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* a,
-                                 const float* b, int n_rows, int W, sd_stream_t stream) {
+extern "C" int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
+                                 const float* c2, const float* a, const float* b, int n_rows, int W,
+                                 sd_stream_t stream) {
   SD_REQUIRE(x && z1 && a && (!b || z2) && n_rows >= 1 && W >= 1, SD_ERR_INVALID, "sd_gated_residual: bad argument");
-  gated_residual_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(x, z1, z2, ldz, a, b, W);
+  gated_residual_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(x, z1, z2, ldz, c1, c2, a, b, W);
   SD_CHECK_LAUNCH("sd_gated_residual");
+  return SD_OK;
+}
+
+extern "C" int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, void* out_bf16, int n_rows,
+                                int F, sd_stream_t stream) {
+  SD_REQUIRE(gate && up && out_bf16 && n_rows >= 1 && F >= 1 && ld >= F, SD_ERR_INVALID,
+             "sd_relu_mul_rows: bad argument");
+  relu_mul_rows_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(gate, up, ld, (bf16_t*)out_bf16, F);
+  SD_CHECK_LAUNCH("sd_relu_mul_rows");
   return SD_OK;
 }
 
@@ -618,19 +644,32 @@ InCols in_cols(const sd_seq_layer& l, int W) {
   return c;
 }
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
+constexpr int kWideRows = 256;  // rows one call of the many-row linear family takes
 struct SeqWs {
-  size_t x, h, proj, dec, o, y, mix, ffo, hout, total;
+  size_t x, h, proj, dec, o, y, mix, ffo, hout, hb, yb, actb, houtb, wide, wide_bytes, total;
 };
 SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
   const int W = m.d.width;
-  size_t proj = 0, hk = 0, hv = 0;
+  size_t proj = 0, hk = 0, hv = 0, ff = 0, wide = 0;
+  const int wr = rows < kWideRows ? rows : kWideRows;
+  auto need = [&](const void* tiled, int M, int N, int K) {
+    if (!tiled || M <= 16) return;
+    const size_t n = sd_linear_wide_workspace_bytes(M, N, K, SD_EPI_F32);
+    wide = n > wide ? n : wide;
+  };
   for (const sd_seq_layer& l : m.layers) {
     const size_t t = in_cols(l, W).total;
     proj = t > proj ? t : proj;
     const size_t a = (size_t)l.heads * l.dim, b = (size_t)l.heads * l.vdim;
     hk = a > hk ? a : hk;
     hv = b > hv ? b : hv;
+    ff = (size_t)l.ff > ff ? (size_t)l.ff : ff;
+    need(l.w_in_tiled, wr, (int)t, W);
+    need(l.w_o_tiled, wr, W, l.heads * l.vdim);
+    need(l.w_down_tiled, wr, W, l.ff);
   }
+  const int no = n_out > 0 ? n_out : 1;
+  need(m.d.head_tiled, no < kWideRows ? no : kWideRows, m.d.vocab, W);
   SeqWs w;
   size_t off = 0;
   const size_t R = (size_t)rows, f = sizeof(float);
@@ -642,9 +681,33 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
   w.y = off;    off += al(R * hv * f);
   w.mix = off;  off += al(R * W * f);
   w.ffo = off;  off += al(R * W * f);
-  w.hout = off; off += al((size_t)(n_out > 0 ? n_out : 1) * W * f);
+  w.hout = off; off += al((size_t)no * W * f);
+  // bf16 copies of the matrix products' operands, for the tiled linear kernels
+  w.hb = off;    off += al(R * W * 2);
+  w.yb = off;    off += al(R * hv * 2);
+  w.actb = off;  off += al(R * (ff ? ff : 1) * 2);
+  w.houtb = off; off += al((size_t)no * W * 2);
+  w.wide_bytes = wide;
+  w.wide = off; off += al(wide ? wide : 16);
   w.total = off;
   return w;
+}
+
+// y[M, N] f32 = x w^T: through the tiled bf16 kernels of the other decoders when the matrix has a
+// tiled copy (x_b: the operand as bf16), else the plain kernel over the row-major matrix.
+int seq_linear(const void* w_rm, const void* w_tiled, int w_f32, const float* x, const float* x2, int64_t ldx,
+               const void* x_b, int64_t ldxb, const float* bias, float* y, int64_t ldy, int M, int N, int K,
+               void* wide_ws, size_t wide_bytes, sd_stream_t stream) {
+  if (!w_tiled) return sd_matmul_rows(x, x2, ldx, w_rm, w_f32, bias, y, ldy, M, N, K, stream);
+  SD_REQUIRE(!bias, SD_ERR_INVALID, "seq_linear: a tiled matrix takes no f32 bias");
+  if (M <= 16) return sd_linear(w_tiled, nullptr, x_b, ldxb, nullptr, nullptr, y, ldy, M, N, K, SD_EPI_F32, stream);
+  for (int r0 = 0; r0 < M; r0 += kWideRows) {
+    const int mm = M - r0 < kWideRows ? M - r0 : kWideRows;
+    const int rc = sd_linear_wide(w_tiled, nullptr, (const bf16_t*)x_b + (size_t)r0 * ldxb, ldxb, nullptr, nullptr,
+                                  y + (size_t)r0 * ldy, ldy, mm, N, K, SD_EPI_F32, wide_ws, wide_bytes, stream);
+    if (rc != SD_OK) return rc;
+  }
+  return SD_OK;
 }
 }  // namespace
 
@@ -663,7 +726,11 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
     const char* bad = nullptr;
     if (l.kind != SD_MIX_HEAD_DECAY && l.kind != SD_MIX_CHANNEL_DECAY && l.kind != SD_MIX_WINDOW_POOL) bad = "unknown mixer";
     else if (l.heads < 1 || l.kv_heads < 1 || l.heads % l.kv_heads || l.dim < 1 || l.vdim < 1) bad = "head counts / sizes";
-    else if (!l.norm_w || !l.w_in || !l.b_in || !l.w_o || (l.ff > 0 && !l.w_down) || l.ff < 0) bad = "a null weight";
+    else if (!l.norm_w || !(l.w_in || l.w_in_tiled) || !(l.w_o || l.w_o_tiled) ||
+             (l.ff > 0 && !(l.w_down || l.w_down_tiled)) || l.ff < 0) bad = "a null weight";
+    else if ((l.w_in_tiled || l.w_o_tiled || l.w_down_tiled) && desc->weights_f32) bad = "tiled matrices are bf16";
+    else if ((l.w_in_tiled && desc->width % 32) || (l.w_o_tiled && (l.heads * l.vdim) % 32) ||
+             (l.w_down_tiled && l.ff % 32)) bad = "a tiled matrix needs an input width that is a multiple of 32";
     else if (l.rot_dims < 0 || l.rot_dims > l.dim || l.rot_dims % 2 || (l.rot_dims && !l.inv_freq)) bad = "rotary dims";
     else if (l.kind == SD_MIX_WINDOW_POOL) {
       if (!l.k_cache || !l.v_cache || !l.pk_cache || !l.pv_cache || l.window < 1 || l.pool < 1 || l.vdim > 256)
@@ -720,6 +787,12 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
   float* ffo = (float*)(base + w.ffo);
   float* hout = (float*)(base + w.hout);
 
+  bf16_t* hb = (bf16_t*)(base + w.hb);
+  bf16_t* yb = (bf16_t*)(base + w.yb);
+  bf16_t* actb = (bf16_t*)(base + w.actb);
+  bf16_t* houtb = (bf16_t*)(base + w.houtb);
+  void* wide_ws = base + w.wide;
+
   if (f32) embed_rows_kernel<float><<<R, 256, 0, st>>>(b->tokens, (const float*)d.embed, x, W, d.vocab);
   else embed_rows_kernel<bf16_t><<<R, 256, 0, st>>>(b->tokens, (const bf16_t*)d.embed, x, W, d.vocab);
   SD_CHECK_LAUNCH("sd_seq_model_forward (embed)");
@@ -729,9 +802,11 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
     const InCols c = in_cols(l, W);
     const int64_t ld = c.total;
     const int H = l.heads, G = l.kv_heads, dk = l.dim, dv = l.vdim;
-    SQ_TRY(sd_rmsnorm_rows(x, nullptr, l.norm_w, f32, 1.f, d.norm_eps, h, R, W, stream));
+    SQ_TRY(sd_rmsnorm_rows(x, nullptr, l.norm_w, f32, 1.f, d.norm_eps, h, l.w_in_tiled ? hb : nullptr, R, W, stream));
     // every matrix that reads h, in one product: q k v g | residual gates | ff gate, up | low-rank decay
-    SQ_TRY(sd_matmul_rows(h, nullptr, W, l.w_in, f32, l.b_in, proj, ld, R, c.total, W, stream));
+    SQ_TRY(seq_linear(l.w_in, l.w_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, ld, R, c.total, W, wide_ws,
+                      w.wide_bytes, stream));
+    bf16_t* y_b = l.w_o_tiled ? yb : nullptr;
     if (l.kind == SD_MIX_WINDOW_POOL) {
       SQ_TRY(sd_head_prep(proj + c.q, proj + c.k, proj + c.v, ld, b->row_pos, b->row_slot, R, H, G, dk, dv,
                           l.rot_dims, l.rot_layout, l.inv_freq, l.qk_unit_norm, d.norm_eps, l.q_scale, l.k_scale,
@@ -739,7 +814,7 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
       SQ_TRY(sd_window_pool_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, l.pk_cache, l.pv_cache,
                                       b->row_pos, b->row_slot, b->block_tables, b->max_blocks, b->page, R, H, G,
                                       dk, dv, l.window, l.pool, l.score_scale, l.head_bias, o, stream));
-      SQ_TRY(sd_head_post(o, proj + c.g, ld, nullptr, f32, 0, d.norm_eps, 1, y, R, H, dv, rnd, stream));
+      SQ_TRY(sd_head_post(o, proj + c.g, ld, nullptr, f32, 0, d.norm_eps, 1, y, y_b, R, H, dv, rnd, stream));
     } else {
       SQ_TRY(sd_head_prep(proj + c.q, proj + c.k, nullptr, ld, b->row_pos, b->row_slot, R, H, H, dk, dv,
                           l.rot_dims, l.rot_layout, l.inv_freq, l.qk_unit_norm, d.norm_eps, l.q_scale, l.k_scale,
@@ -753,13 +828,17 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
       }
       SQ_TRY(sd_decay_scan(proj + c.q, proj + c.k, proj + c.v, ld, pc ? dec : l.head_decay, pc, l.state,
                            b->entries, b->n_entries, o, H, dk, dv, stream));
-      SQ_TRY(sd_head_post(o, proj + c.g, ld, l.head_norm_w, f32, 1, d.norm_eps, 0, y, R, H, dv, rnd, stream));
+      SQ_TRY(sd_head_post(o, proj + c.g, ld, l.head_norm_w, f32, 1, d.norm_eps, 0, y, y_b, R, H, dv, rnd, stream));
     }
-    SQ_TRY(sd_matmul_rows(y, nullptr, (int64_t)H * dv, l.w_o, f32, nullptr, mix, W, R, W, H * dv, stream));
-    if (l.ff > 0)
-      SQ_TRY(sd_matmul_rows(proj + c.gate, proj + c.up, ld, l.w_down, f32, nullptr, ffo, W, R, W, l.ff, stream));
-    SQ_TRY(sd_gated_residual(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, mix, l.ff > 0 ? ffo : nullptr,
-                             R, W, stream));
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, y, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R,
+                      W, H * dv, wide_ws, w.wide_bytes, stream));
+    if (l.ff > 0) {
+      if (l.w_down_tiled) SQ_TRY(sd_relu_mul_rows(proj + c.gate, proj + c.up, ld, actb, R, l.ff, stream));
+      SQ_TRY(seq_linear(l.w_down, l.w_down_tiled, f32, proj + c.gate, proj + c.up, ld, actb, l.ff, nullptr, ffo, W,
+                        R, W, l.ff, wide_ws, w.wide_bytes, stream));
+    }
+    SQ_TRY(sd_gated_residual(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, l.r1_bias,
+                             l.ff > 0 ? l.r2_bias : nullptr, mix, l.ff > 0 ? ffo : nullptr, R, W, stream));
     if (b->layer_out) {
       const hipError_t e = hipMemcpyAsync(b->layer_out + (size_t)li * R * W, x, (size_t)R * W * sizeof(float),
                                           hipMemcpyDeviceToDevice, st);
@@ -768,8 +847,10 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
     }
   }
   if (b->n_out > 0) {
-    SQ_TRY(sd_rmsnorm_rows(x, b->out_rows, d.final_norm_w, f32, 1.f, d.norm_eps, hout, b->n_out, W, stream));
-    SQ_TRY(sd_matmul_rows(hout, nullptr, W, d.embed, f32, nullptr, b->logits, d.vocab, b->n_out, d.vocab, W, stream));
+    SQ_TRY(sd_rmsnorm_rows(x, b->out_rows, d.final_norm_w, f32, 1.f, d.norm_eps, hout,
+                           d.head_tiled ? houtb : nullptr, b->n_out, W, stream));
+    SQ_TRY(seq_linear(d.embed, d.head_tiled, f32, hout, nullptr, W, houtb, W, nullptr, b->logits, d.vocab, b->n_out,
+                      d.vocab, W, wide_ws, w.wide_bytes, stream));
   }
   return SD_OK;
 }

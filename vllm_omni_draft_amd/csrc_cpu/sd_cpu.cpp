@@ -1465,8 +1465,8 @@ extern "C" int sd_debug_force_proposals(int32_t* tok_buf, int k, const int32_t* 
 // ---------------------------------------------------------------- sequence mixers: GPU library only
 extern "C" int sd_matmul_rows(const float*, const float*, int64_t, const void*, int, const float*, float*,
                               int64_t, int, int, int, sd_stream_t) { UNSUPPORTED("sd_matmul_rows"); }
-extern "C" int sd_rmsnorm_rows(const float*, const int32_t*, const void*, int, float, float, float*, int, int,
-                               sd_stream_t) { UNSUPPORTED("sd_rmsnorm_rows"); }
+extern "C" int sd_rmsnorm_rows(const float*, const int32_t*, const void*, int, float, float, float*, void*, int,
+                               int, sd_stream_t) { UNSUPPORTED("sd_rmsnorm_rows"); }
 extern "C" int sd_head_prep(float*, float*, const float*, int64_t, const int32_t*, const int32_t*, int, int, int,
                             int, int, int, int, const double*, int, float, float, float, void*, void*, int,
                             const int32_t*, int, int, sd_stream_t) { UNSUPPORTED("sd_head_prep"); }
@@ -1475,16 +1475,19 @@ extern "C" int sd_sigmoid_power(const float*, int64_t, float, float*, int, int, 
 }
 extern "C" int sd_decay_scan(const float*, const float*, const float*, int64_t, const float*, int, float*,
                              const int32_t*, int, float*, int, int, int, sd_stream_t) { UNSUPPORTED("sd_decay_scan"); }
-extern "C" int sd_head_post(const float*, const float*, int64_t, const void*, int, int, float, int, float*, int,
-                            int, int, int, sd_stream_t) { UNSUPPORTED("sd_head_post"); }
+extern "C" int sd_head_post(const float*, const float*, int64_t, const void*, int, int, float, int, float*, void*,
+                            int, int, int, int, sd_stream_t) { UNSUPPORTED("sd_head_post"); }
 extern "C" int sd_pooled_slots_per_page(int page, int pool) { return page < 1 || pool < 1 ? 0 : page / pool + 2; }
 extern "C" int sd_window_pool_attention(const float*, int64_t, const void*, const void*, int, float*, float*,
                                         const int32_t*, const int32_t*, const int32_t*, int, int, int, int, int,
                                         int, int, int, int, float, const float*, float*, sd_stream_t) {
   UNSUPPORTED("sd_window_pool_attention");
 }
-extern "C" int sd_gated_residual(float*, const float*, const float*, int64_t, const float*, const float*, int,
-                                 int, sd_stream_t) { UNSUPPORTED("sd_gated_residual"); }
+extern "C" int sd_gated_residual(float*, const float*, const float*, int64_t, const float*, const float*,
+                                 const float*, const float*, int, int, sd_stream_t) { UNSUPPORTED("sd_gated_residual"); }
+extern "C" int sd_relu_mul_rows(const float*, const float*, int64_t, void*, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_relu_mul_rows");
+}
 extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc*) {
   set_error("sd_seq_model_create: not provided by the CPU build of the library");
   return nullptr;

@@ -220,6 +220,13 @@ class SeqModel:
         cfg = self.cfg
         f32 = weights.dtype == torch.float32
         layers = (_lib.SeqLayer * cfg.n_layers)()
+
+        def rm(w):   # a row-major matrix, or nothing
+            return None if w is None or isinstance(w, ops.TiledWeight) else w.data_ptr()
+
+        def tl(w):   # a tiled matrix, or nothing
+            return w.data.data_ptr() if isinstance(w, ops.TiledWeight) else None
+
         for i, (spec, t) in enumerate(zip(cfg.layers, weights.layers)):
             m = spec.mixer
             rec = m.kind != "attention"
@@ -230,8 +237,9 @@ class SeqModel:
                 q_scale=m.dim ** -0.5 if m.kind == "gla" else 1.0,
                 k_scale=m.dim ** -0.5 if m.kind == "retention" else 1.0,
                 score_scale=m.scale, window=m.window, pool=m.pool, rank=m.rank, tau=m.tau,
-                norm_w=_ptr(t.norm_w), w_in=_ptr(t.w_in), b_in=_ptr(t.b_in), w_o=_ptr(t.w_o),
-                w_down=_ptr(t.w_down), w_a2=_ptr(t.w_a2), b_a2=_ptr(t.b_a2),
+                norm_w=_ptr(t.norm_w), w_in=rm(t.w_in), w_in_tiled=tl(t.w_in), r1_bias=_ptr(t.r1_bias),
+                r2_bias=_ptr(t.r2_bias), w_o=rm(t.w_o), w_o_tiled=tl(t.w_o), w_down=rm(t.w_down),
+                w_down_tiled=tl(t.w_down), w_a2=_ptr(t.w_a2), b_a2=_ptr(t.b_a2),
                 head_decay=_ptr(t.head_decay), head_bias=_ptr(t.head_bias),
                 head_norm_w=_ptr(t.head_norm_w),
                 state=_ptr(cache.state.get(i)) if rec else None,
@@ -239,7 +247,7 @@ class SeqModel:
                 pk_cache=_ptr(cache.pk.get(i)), pv_cache=_ptr(cache.pv.get(i)))
         desc = _lib.SeqModelDesc(n_layers=cfg.n_layers, width=cfg.width, vocab=cfg.vocab,
                                  weights_f32=int(f32), norm_eps=cfg.norm_eps, embed=_ptr(weights.embed),
-                                 final_norm_w=_ptr(weights.final_norm_w), layers=layers)
+                                 head_tiled=tl(weights.head_tiled), final_norm_w=_ptr(weights.final_norm_w), layers=layers)
         self._handle = _lib.load().sd_seq_model_create(C.byref(desc))
         if not self._handle:
             raise _lib.SdError(f"sd_seq_model_create failed: {_lib.last_error()}")

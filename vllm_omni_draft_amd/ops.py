@@ -1065,13 +1065,15 @@ def matmul_rows(x: torch.Tensor, w: torch.Tensor, bias=None, x2=None) -> torch.T
     return y
 
 
-def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, offset: float = 0.0, rows=None) -> torch.Tensor:
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, offset: float = 0.0, rows=None,
+                 bf16_copy: bool = False):
     _f32(x, "x")
     n = x.shape[0] if rows is None else rows.numel()
     out = torch.empty(n, x.shape[1], dtype=torch.float32, device=x.device)
+    out_b = torch.empty(n, x.shape[1], dtype=torch.bfloat16, device=x.device) if bf16_copy else None
     _lib.check(_lib.load().sd_rmsnorm_rows(_p(x), _p(rows), _p(w), _wkind(w, "w"), float(offset), float(eps),
-                                           _p(out), n, x.shape[1], _stream()), "sd_rmsnorm_rows")
-    return out
+                                           _p(out), _p(out_b), n, x.shape[1], _stream()), "sd_rmsnorm_rows")
+    return (out, out_b) if bf16_copy else out
 
 
 def head_prep(q, k, row_pos, Hq, Hk, dk, *, rot_dims=0, rot_layout=0, inv_freq=None, unit_norm=False,
@@ -1119,15 +1121,17 @@ def decay_scan(q, k, v, decay, state, entries, H, dk, dv) -> torch.Tensor:
     return out
 
 
-def head_post(o, g, H, dv, *, norm_w=None, unit_norm=False, eps=1e-5, gate="silu", round_bf16=False):
+def head_post(o, g, H, dv, *, norm_w=None, unit_norm=False, eps=1e-5, gate="silu", round_bf16=False,
+              bf16_copy=False):
     _f32(o, "o")
     _f32(g, "g")
     y = torch.empty_like(o)
+    y_b = torch.empty_like(o, dtype=torch.bfloat16) if bf16_copy else None
     _lib.check(_lib.load().sd_head_post(_p(o), _p(g), g.shape[1], _p(norm_w),
                                         _wkind(norm_w, "norm_w") if norm_w is not None else 1, int(unit_norm),
-                                        float(eps), {"silu": 0, "sigmoid": 1}[gate], _p(y), o.shape[0], H, dv,
-                                        int(round_bf16), _stream()), "sd_head_post")
-    return y
+                                        float(eps), {"silu": 0, "sigmoid": 1}[gate], _p(y), _p(y_b), o.shape[0],
+                                        H, dv, int(round_bf16), _stream()), "sd_head_post")
+    return (y, y_b) if bf16_copy else y
 
 
 def window_pool_attention(q, k_cache, v_cache, pk_cache, pv_cache, row_pos, row_slot, block_tables, H, G,
@@ -1143,9 +1147,20 @@ def window_pool_attention(q, k_cache, v_cache, pk_cache, pv_cache, row_pos, row_
     return out
 
 
-def gated_residual(x, z1, a, z2=None, b=None) -> None:
-    """x += sigmoid(z1) * a (+ sigmoid(z2) * b), in place; all f32 [rows, W]."""
+def gated_residual(x, z1, a, z2=None, b=None, c1=None, c2=None) -> None:
+    """x += sigmoid(z1 + c1) * a (+ sigmoid(z2 + c2) * b), in place; x, z, a, b f32 [rows, W],
+    the bias rows c1, c2 f32 [W]."""
     for t, nm in ((x, "x"), (z1, "z1"), (a, "a")):
         _f32(t, nm)
-    _lib.check(_lib.load().sd_gated_residual(_p(x), _p(z1), _p(z2), x.shape[1], _p(a), _p(b), x.shape[0],
-                                             x.shape[1], _stream()), "sd_gated_residual")
+    _lib.check(_lib.load().sd_gated_residual(_p(x), _p(z1), _p(z2), x.shape[1], _p(c1), _p(c2), _p(a), _p(b),
+                                             x.shape[0], x.shape[1], _stream()), "sd_gated_residual")
+
+
+def relu_mul_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """bf16(relu(gate) * up) for f32 [rows, F] inputs."""
+    _f32(gate, "gate")
+    _f32(up, "up")
+    out = torch.empty(gate.shape, dtype=torch.bfloat16, device=gate.device)
+    _lib.check(_lib.load().sd_relu_mul_rows(_p(gate), _p(up), gate.shape[1], _p(out), gate.shape[0],
+                                            gate.shape[1], _stream()), "sd_relu_mul_rows")
+    return out

@@ -321,10 +321,13 @@ def from_safetensors_dir(cfg: ModelConfig, model_dir: str, device="cuda",
 @dataclass
 class SeqLayerTensors:
     norm_w: torch.Tensor
-    w_in: torch.Tensor            # [q | k | v | g | r1 | r2 | ff gate | ff up | a1] x width
-    b_in: torch.Tensor            # f32 bias of w_in (the residual gates' biases; zero elsewhere)
-    w_o: torch.Tensor
-    w_down: Optional[torch.Tensor] = None
+    # A matrix is either a row-major tensor or, for bfloat16 serving and an input width that is a
+    # multiple of 32, an ops.TiledWeight for the MFMA linear kernels the other decoders use.
+    w_in: object                  # [q | k | v | g | r1 | r2 | ff gate | ff up | a1] x width
+    w_o: object
+    r1_bias: torch.Tensor         # f32 [width]
+    r2_bias: Optional[torch.Tensor] = None
+    w_down: object = None
     w_a2: Optional[torch.Tensor] = None
     b_a2: Optional[torch.Tensor] = None       # f32
     head_decay: Optional[torch.Tensor] = None  # f32 [heads]
@@ -340,13 +343,18 @@ class SeqModelWeights:
     embed: torch.Tensor
     final_norm_w: torch.Tensor
     layers: List[SeqLayerTensors]
+    head_tiled: Optional["ops.TiledWeight"] = None   # the embedding table once more, tiled, as the head
 
     def tensors(self):
         yield self.embed
         yield self.final_norm_w
+        if self.head_tiled is not None:
+            yield self.head_tiled.data
         for l in self.layers:
             for t in vars(l).values():
-                if t is not None:
+                if isinstance(t, ops.TiledWeight):
+                    yield t.data
+                elif t is not None:
                     yield t
 
     def nbytes(self) -> int:
@@ -354,9 +362,10 @@ class SeqModelWeights:
 
 
 def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
-                        dtype: torch.dtype = torch.bfloat16) -> SeqModelWeights:
+                        dtype: torch.dtype = torch.bfloat16, tiled: bool = True) -> SeqModelWeights:
     """Tensors under the checkpoint's names ('embed', 'final.norm', 'l<i>.norm1', 'l<i>.mix.*',
-    'l<i>.mlp.*', 'l<i>.rg1', 'l<i>.rg1.b', ...) -> device tensors in the serving dtype."""
+    'l<i>.mlp.*', 'l<i>.rg1', 'l<i>.rg1.b', ...) -> device tensors in the serving dtype.
+    tiled=False keeps every matrix row-major (the plain kernels), whatever its shape."""
     if dtype not in (torch.bfloat16, torch.float32):
         raise ValueError("a layer-list model is served in bfloat16 or float32")
     W = cfg.width
@@ -372,24 +381,29 @@ def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
     def dev(t, dt=None):
         return t.to(dt or dtype).contiguous().to(device)
 
+    def mat(t):
+        """A matrix [N, K] for the linear layers."""
+        d = dev(t)
+        if tiled and dtype == torch.bfloat16 and t.shape[1] % 32 == 0 and torch.device(device).type == "cuda":
+            return ops.tile_weights(d, ops.TILE_PLAIN)
+        return d
+
     layers = []
     for i, l in enumerate(cfg.layers):
         m, p = l.mixer, f"l{i}."
         H, G, dk, dv = m.heads, m.kv_heads, m.dim, m.vdim
         parts = [get(p + "mix.q", (H * dk, W)), get(p + "mix.k", (G * dk, W)), get(p + "mix.v", (G * dv, W)),
                  get(p + "mix.g", (H * dv, W)), get(p + "rg1", (W, W))]
-        bias = [torch.zeros(H * dk + G * dk + G * dv + H * dv), get(p + "rg1.b", (W,)).float()]
         if l.ff:
             parts += [get(p + "rg2", (W, W)), get(p + "mlp.gate", (l.ff, W)), get(p + "mlp.up", (l.ff, W))]
-            bias += [get(p + "rg2.b", (W,)).float(), torch.zeros(2 * l.ff)]
         if m.kind == "gla":
             parts.append(get(p + "mix.a1", (m.rank, W)))
-            bias.append(torch.zeros(m.rank))
         lt = SeqLayerTensors(
-            norm_w=dev(get(p + "norm1", (W,))), w_in=dev(torch.cat([t.float() for t in parts])),
-            b_in=dev(torch.cat(bias), torch.float32), w_o=dev(get(p + "mix.o", (W, H * dv))))
+            norm_w=dev(get(p + "norm1", (W,))), w_in=mat(torch.cat([t.float() for t in parts])),
+            w_o=mat(get(p + "mix.o", (W, H * dv))), r1_bias=dev(get(p + "rg1.b", (W,)), torch.float32))
         if l.ff:
-            lt.w_down = dev(get(p + "mlp.down", (W, l.ff)))
+            lt.w_down = mat(get(p + "mlp.down", (W, l.ff)))
+            lt.r2_bias = dev(get(p + "rg2.b", (W,)), torch.float32)
         if m.kind == "gla":
             lt.w_a2 = dev(get(p + "mix.a2", (H * dk, m.rank)))
             lt.b_a2 = dev(get(p + "mix.a2.b", (H * dk,)), torch.float32)
@@ -403,7 +417,10 @@ def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
             lt.inv_freq = dev(torch.tensor(m.rot_base, dtype=torch.float64) ** (-2.0 * i2 / m.rot_dims),
                               torch.float64)
         layers.append(lt)
-    return SeqModelWeights(cfg, dtype, dev(get("embed", (cfg.vocab, W))), dev(get("final.norm", (W,))), layers)
+    embed = dev(get("embed", (cfg.vocab, W)))
+    head = mat(get("embed", (cfg.vocab, W)))
+    return SeqModelWeights(cfg, dtype, embed, dev(get("final.norm", (W,))), layers,
+                           head if isinstance(head, ops.TiledWeight) else None)
 
 
 def seq_from_safetensors_dir(cfg, model_dir: str, device="cuda",
