@@ -102,6 +102,12 @@ def parse():
     ap.add_argument("--tp-draft", choices=["replicated", "sharded"], default="replicated",
                     help="the draft whole on every rank (no exchange in its passes), or sharded "
                          "like the target with a vocabulary-parallel head")
+    ap.add_argument("--family", choices=["spec", "puguzen"], default="spec",
+                    help="spec: the headline speculative-decoding workload (default).  puguzen: prefill and "
+                         "decode throughput of the Puguzen decoder family (recurrent and windowed layers) at "
+                         "layer sizes of real models, beside a Llama-style decoder of equal size, with the "
+                         "time and memory traffic of its own kernels")
+    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen: sizes to run")
     return ap.parse_args()
 
 
@@ -626,8 +632,177 @@ def main_tp(args):
     dist.destroy_process_group()
 
 
+# ---------------------------------------------------------------------------------------------
+# --family puguzen
+SEQ_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, ff=4096),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, ff=8192),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, ff=14336),
+}
+SEQ_HEAD, SEQ_VOCAB, SEQ_WINDOW, SEQ_POOL, SEQ_RANK = 128, 32000, 1024, 16, 64
+
+
+def _seq_config(sz):
+    from vllm_omni_draft_amd.config import MixerSpec, SeqLayerSpec, SeqModelConfig
+    H, G, D = sz["heads"], sz["kv_heads"], SEQ_HEAD
+    rot = dict(rot_dims=D, rot_base=1e6)
+    ret = MixerSpec("retention", H, D, D, decay=tuple(1 - 2.0 ** (-5 - 3 * i / H) for i in range(H)), **rot)
+    att = MixerSpec("attention", H, D, D, kv_heads=G, rot_layout="interleaved", scale=D ** -0.5,
+                    window=SEQ_WINDOW, pool=SEQ_POOL, **rot)
+    gla = MixerSpec("gla", H, D, D, tau=16.0, rank=SEQ_RANK)
+    cfg = SeqModelConfig("puguzen", sz["width"], SEQ_VOCAB,
+                         [SeqLayerSpec(m, sz["ff"]) for m in (ret, att, gla, att)], name="puguzen-bench")
+    cfg.validate()
+    return cfg
+
+
+def _events(fn, reps):
+    fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps      # microseconds
+
+
+def seq_kernel_rooflines(cfg, device, ctx, rows):
+    """The family's own kernels alone, at `rows` token rows of one sequence whose first row sits at
+    position ctx - rows: time, the bytes each must move at least, and the fraction of the HBM
+    peak that makes.  (The linear layers are the tiled kernels the Llama-style decoder runs.)"""
+    from vllm_omni_draft_amd import ops
+    att = next(l.mixer for l in cfg.layers if l.mixer.kind == "attention")
+    rec = next(l.mixer for l in cfg.layers if l.mixer.kind == "retention")
+    H, G, D = att.heads, att.kv_heads, att.dim
+    g = torch.Generator(device="cpu").manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g).to(device)
+    out = []
+    # decayed recurrence (per head and per channel)
+    q, k, v = rn(rows, H * D), rn(rows, H * D) * D ** -0.5, rn(rows, H * D)
+    state = torch.zeros(1, H, D, D, device=device)
+    ent = torch.tensor([[0, 0, rows, 1]], dtype=torch.int32, device=device)
+    for name, dec in (("decay_scan (decay per head)", torch.full((H,), 0.97, device=device)),
+                      ("decay_scan (decay per channel)", torch.rand(rows, H * D, generator=g).to(device) * 0.1 + 0.9)):
+        us = _events(lambda: ops.decay_scan(q, k, v, dec, state, ent, H, D, D), 5)
+        nbytes = 4 * (rows * H * D * (4 + (dec.dim() == 2)) + 2 * H * D * D)
+        out.append((name, us, nbytes))
+    # window attention with pooled blocks over a filled cache
+    pages = -(-ctx // ops.PAGE)
+    kc = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    vc = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    ps = ops.pooled_slots_per_page(ops.PAGE, att.pool)
+    pk, pv = torch.zeros(pages, G, ps, D, device=device), torch.zeros(pages, G, ps, D, device=device)
+    tables = torch.arange(pages, dtype=torch.int32, device=device).view(1, -1)
+    pos = torch.arange(ctx - rows, ctx, dtype=torch.int32, device=device)
+    slot = torch.zeros(rows, dtype=torch.int32, device=device)
+    qa = rn(rows, H * D)
+    bias = torch.full((H,), -4.0, device=device)
+    us = _events(lambda: ops.window_pool_attention(qa, kc, vc, pk, pv, pos, slot, tables, H, G, D, D, att.window,
+                                                   att.pool, att.scale, bias), 5)
+    keys = min(ctx, att.window + rows - 1)
+    nbytes = G * 2 * D * (2 * keys + 4 * (ctx // att.pool)) + 8 * rows * H * D
+    out.append(("window_pool_attention", us, nbytes))
+    res = []
+    for name, us, nbytes in out:
+        gbs = nbytes / us * 1e-3
+        res.append({"kernel": name, "rows": rows, "ctx": ctx, "avg_us": round(us, 2), "min_bytes": int(nbytes),
+                    "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
+    return res
+
+
+def main_seq_family(args):
+    """Prefill and decode throughput of the Puguzen family beside a Llama-style decoder of equal
+    width, heads, feed-forward and depth (both bf16, seeded random weights), one JSON line."""
+    from vllm_omni_draft_amd import config, weights
+    from vllm_omni_draft_amd.engine import EngineConfig, SpecEngine
+    from vllm_omni_draft_amd.seq_engine import SeqEngine, SeqEngineConfig
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (there is no CPU path)")
+    device = torch.device("cuda", 0)
+    P, B, steps, warm = args.prompt_len, 4, args.steps, args.warmup
+    results = []
+    for name in args.seq_sizes.split(","):
+        sz = SEQ_SIZES[name]
+        cfg = _seq_config(sz)
+        w = weights.seq_from_state_dict(cfg, weights.seq_random_state(cfg, 0), device, torch.bfloat16)
+        g = torch.Generator().manual_seed(7)
+        prompts = [torch.randint(0, SEQ_VOCAB, (P,), generator=g).tolist() for _ in range(B)]
+        eng = SeqEngine(w, SeqEngineConfig(max_seqs=B, max_tokens=B * (P + steps + warm + 64), max_rows=2048,
+                                           max_seq_len=P + steps + warm + 64))
+        eng.step([("warm", prompts[0][:300], [299])])
+        eng.finish("warm")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        first = eng.step([("s0", prompts[0], [P - 1])])
+        torch.cuda.synchronize()
+        prefill_s = time.perf_counter() - t0
+        for i in range(1, B):
+            eng.step([(f"s{i}", prompts[i], [P - 1])])
+        toks = [1] * B
+
+        def decode(n):
+            nonlocal toks
+            for _ in range(n):
+                lg = eng.step([(f"s{i}", [toks[i]], [0]) for i in range(B)])
+                toks = lg.argmax(-1).tolist()        # one read-back per step, like a serving loop
+        decode(warm)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        decode(steps)
+        torch.cuda.synchronize()
+        decode_s = time.perf_counter() - t0
+        kern = seq_kernel_rooflines(cfg, device, P, 1) + seq_kernel_rooflines(cfg, device, P, min(P, 1024))
+        seq_bytes = w.nbytes()
+        del eng, w
+        torch.cuda.empty_cache()
+        # the closest existing decoder at equal size
+        lc = config.create_model_config(None, arch="llama", n_layers=cfg.n_layers, hidden=sz["width"],
+                                        n_heads=sz["heads"], n_kv_heads=sz["kv_heads"], head_dim=SEQ_HEAD,
+                                        ffn=sz["ff"], vocab=SEQ_VOCAB, max_pos=P + steps + warm + 128, name="llama-equal")
+        lw = weights.random_init(lc, seed=0, device=device)
+        ar = SpecEngine(lw, None, EngineConfig(k=0, max_batch=B, max_seq_len=P + steps + warm + 64, rows="narrow",
+                                               gen_capacity=steps + warm + 64, use_graph=False))
+        ar.add_request(0, prompts[0][:300])
+        ar.remove_request(0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ar.add_request(0, prompts[0])
+        torch.cuda.synchronize()
+        l_prefill_s = time.perf_counter() - t0
+        for i in range(1, B):
+            ar.add_request(i, prompts[i])
+        for _ in range(warm):
+            ar.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ar.step()
+        torch.cuda.synchronize()
+        l_decode_s = time.perf_counter() - t0
+        del ar
+        results.append({
+            "size": name, **sz, "layers": [l.mixer.kind for l in cfg.layers], "head_dim": SEQ_HEAD,
+            "window": SEQ_WINDOW, "pool": SEQ_POOL, "prompt_len": P, "decode_batch": B,
+            "puguzen": {"weight_bytes": seq_bytes, "prefill_tokens_per_s": round(P / prefill_s, 1),
+                        "decode_tokens_per_s": round(B * steps / decode_s, 1),
+                        "decode_ms_per_step": round(decode_s / steps * 1e3, 3)},
+            "llama_equal_size": {"weight_bytes": lw.nbytes(), "prefill_tokens_per_s": round(P / l_prefill_s, 1),
+                                 "decode_tokens_per_s": round(B * steps / l_decode_s, 1),
+                                 "decode_ms_per_step": round(l_decode_s / steps * 1e3, 3)},
+            "kernels": kern})
+        del lw
+        torch.cuda.empty_cache()
+        _ = first
+    print(json.dumps({"metric": "puguzen_family_throughput", "unit": "tokens/s", "dtype": "bf16",
+                      "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
+
+
 def main():
     args = parse()
+    if args.family == "puguzen":
+        main_seq_family(args)
+        return
     if args.cpu_baseline_worker:
         cpu_baseline_worker(args.cpu_budget)
         return

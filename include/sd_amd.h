@@ -1081,13 +1081,19 @@ int sd_pooled_slots_per_page(int page, int pool);
  * b*pool .. b*pool+pool-1) once b*pool + pool - 1 <= i - window, as the mean of its cached keys
  * and of its values (pk_cache / pv_cache, f32, sd_pooled_slots_per_page entries per page and
  * head; computed here when a row completes a block).  out[r, h] = sum over visible keys of
- * sigmoid(q.k * scale + head_bias[h]) * v; query head h reads kv head h / (H/G).  dv <= 256. */
+ * sigmoid(q.k * scale + head_bias[h]) * v; query head h reads kv head h / (H/G).  dv <= 256.
+ * scratch (may be NULL): sd_window_pool_attention_scratch_bytes(n_rows, ..., max_blocks * page)
+ * bytes let a batch of few rows cut each row's keys into tiles that run as workgroups of their
+ * own (their sums are added in tile order); 0 bytes means that no such cut would be made.   */
+size_t sd_window_pool_attention_scratch_bytes(int n_rows, int H, int dv, int window, int pool,
+                                              int max_ctx);
 int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
                              int cache_f32, float* pk_cache, float* pv_cache,
                              const int32_t* row_pos, const int32_t* row_slot,
                              const int32_t* block_tables, int max_blocks, int page, int n_rows,
                              int H, int G, int dk, int dv, int window, int pool, float scale,
-                             const float* head_bias, float* out, sd_stream_t stream);
+                             const float* head_bias, float* out, void* scratch, size_t scratch_bytes,
+                             sd_stream_t stream);
 /* x += sigmoid(z1 + c1) * a + sigmoid(z2 + c2) * b (b, z2 and the bias rows c1, c2 [W] may be
  * NULL); x, a, b [rows, W].                                                                */
 int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
@@ -1170,7 +1176,7 @@ typedef struct {
 typedef struct sd_seq_model sd_seq_model;
 sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc);
 void sd_seq_model_destroy(sd_seq_model* m);
-size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out);
+size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out, int max_ctx);
 /* One pass over a ragged batch: enqueues kernels only.                                     */
 int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* batch, void* workspace,
                          size_t workspace_bytes, sd_stream_t stream);

@@ -278,6 +278,32 @@ def test_window_pool_attention_random(H, G, dk, dv, window, pool, step):
             assert rel(out[i, h], w @ Vt[:, gi]) < 5e-6, (i, h)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_window_pool_attention_many_keys(dtype):
+    """More visible keys than one tile of the kernel holds: rows in small batches (their keys are
+    cut over several workgroups) and in large ones (one workgroup walks the tiles) agree with the
+    plain sum and with each other."""
+    g = torch.Generator().manual_seed(5)
+    H, G, dk, dv, window, pool, n = 4, 2, 32, 48, 300, 2, 700
+    rd = (lambda t: t.to(torch.bfloat16).float()) if dtype == torch.bfloat16 else (lambda t: t)
+    k, v = rd(torch.randn(n, G * dk, generator=g)), rd(torch.randn(n, G * dv, generator=g))
+    q, bias = torch.randn(n, H * dk, generator=g), torch.randn(H, generator=g) - 3
+    bed = _AttnBed(G, dk, dv, pool, n, dtype)
+    bed.append(k, v, list(range(n)))
+    big = bed.attend(q, list(range(n)), H, window, 0.2, bias).cpu()           # 700 rows: no cut
+    rows = [5, 255, 256, 257, 299, 300, 301, 511, 512, 640, 699]
+    small = bed.attend(q[rows], rows, H, window, 0.2, bias).cpu()             # 11 rows: keys cut into tiles
+    K, V, Q = k.double().view(n, G, dk), v.double().view(n, G, dv), q.double().view(n, H, dk)
+    for a, i in enumerate(rows):
+        toks, blocks = P.visible_keys(i, window, pool)
+        Kt = torch.stack([K[j] for j in toks] + [K[b * pool:(b + 1) * pool].mean(0) for b in blocks])
+        Vt = torch.stack([V[j] for j in toks] + [V[b * pool:(b + 1) * pool].mean(0) for b in blocks])
+        for h in range(H):
+            w = torch.sigmoid(Kt[:, h // 2] @ Q[i, h] * 0.2 + bias[h].double())
+            ref = w @ Vt[:, h // 2]
+            assert rel(small[a].view(H, dv)[h], ref) < 5e-6 and rel(big[i].view(H, dv)[h], ref) < 5e-6, (i, h)
+
+
 @pytest.mark.parametrize("window,pool", [(9, 4), (7, 5), (16, 16), (17, 3), (1, 1), (5, 32)])
 @pytest.mark.parametrize("decode", [False, True])
 def test_window_pool_attention_sees_exactly_its_keys(window, pool, decode):

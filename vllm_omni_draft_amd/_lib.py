@@ -218,13 +218,14 @@ SIGNATURES = {
     "sd_decay_scan": (i32, [vp, vp, vp, i64, vp, i32, vp, vp, i32, vp, i32, i32, i32, vp]),
     "sd_head_post": (i32, [vp, vp, i64, vp, i32, i32, C.c_float, i32, vp, vp, i32, i32, i32, i32, vp]),
     "sd_pooled_slots_per_page": (i32, [i32, i32]),
+    "sd_window_pool_attention_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32, i32]),
     "sd_window_pool_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
-                                       i32, i32, i32, C.c_float, vp, vp, vp]),
+                                       i32, i32, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]),
     "sd_gated_residual": (i32, [vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, vp]),
     "sd_relu_mul_rows": (i32, [vp, vp, i64, vp, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),
-    "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32]),
+    "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32, i32]),
     "sd_seq_model_forward": (i32, [vp, C.POINTER(SeqBatch), vp, C.c_size_t, vp]),
     "sd_graph_destroy": (None, [vp]),
 }

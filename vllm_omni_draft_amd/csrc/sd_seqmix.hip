@@ -215,6 +215,8 @@ __global__ void sigmoid_power_kernel(const float* __restrict__ z, int64_t ldz, f
 // 16 consecutive key channels of one value column; the strips' partial dot products are added in
 // strip order.  d_t: a factor per key channel (PER_CHANNEL, [rows, H*dk]) or per head ([H]).
 constexpr int kStrip = 16;
+constexpr int kScanLoads = 8;    // q / k / decay elements a thread stages per chunk, at most
+constexpr int kScanLoadsV = 16;  // value elements
 template <bool PER_CHANNEL>
 __global__ __launch_bounds__(256) void decay_scan_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, int64_t ld,
@@ -240,22 +242,49 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
   for (int r = 0; r < kStrip; ++r)
     S[r] = (pos0 > 0 && r0 + r < dk && col < dv) ? st[(size_t)(r0 + r) * dv + col] : 0.f;
   const float dh = PER_CHANNEL ? 0.f : decay[h];
+  // A chunk of CH tokens goes global -> registers -> LDS; the next chunk's loads are in flight
+  // while this one is computed.
+  float pq[kScanLoads], pk[kScanLoads], pd[kScanLoads], pv[kScanLoadsV];
+  auto fetch = [&](int t0) {
+    const int nt = len - t0 < CH ? len - t0 : CH;
+#pragma unroll
+    for (int i = 0; i < kScanLoads; ++i) {
+      const int idx = tid + i * nthr;
+      const int t = idx / dkp, ch = idx % dkp;
+      const bool in = idx < nt * dkp && ch < dk;
+      const size_t at = (size_t)(row0 + t0 + (in ? t : 0)) * ld + (size_t)h * dk + (in ? ch : 0);
+      pq[i] = in ? q[at] : 0.f;
+      pk[i] = in ? k[at] : 0.f;
+      if (PER_CHANNEL)
+        pd[i] = in ? decay[(size_t)(row0 + t0 + t) * ((size_t)H * dk) + (size_t)h * dk + ch] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < kScanLoadsV; ++i) {
+      const int idx = tid + i * nthr;
+      const int t = idx / CT, vcol = blockIdx.x * CT + idx % CT;
+      const bool in = idx < nt * CT && vcol < dv;
+      pv[i] = in ? v[(size_t)(row0 + t0 + t) * ld + (size_t)h * dv + vcol] : 0.f;
+    }
+  };
+  fetch(0);
   for (int t0 = 0; t0 < len; t0 += CH) {
     const int nt = len - t0 < CH ? len - t0 : CH;
-    for (int idx = tid; idx < nt * dkp; idx += nthr) {
-      const int t = idx / dkp, ch = idx % dkp;
-      const size_t row = (size_t)(row0 + t0 + t);
-      const bool in = ch < dk;
-      qs[t * dkp + ch] = in ? q[row * ld + (size_t)h * dk + ch] : 0.f;
-      ks[t * dkp + ch] = in ? k[row * ld + (size_t)h * dk + ch] : 0.f;
-      if (PER_CHANNEL) ds[t * dkp + ch] = in ? decay[row * ((size_t)H * dk) + (size_t)h * dk + ch] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kScanLoads; ++i) {
+      const int idx = tid + i * nthr;
+      if (idx < CH * dkp) {
+        qs[idx] = pq[i];
+        ks[idx] = pk[i];
+        if (PER_CHANNEL) ds[idx] = pd[i];
+      }
     }
-    for (int idx = tid; idx < nt * CT; idx += nthr) {
-      const int t = idx / CT, cc = idx % CT;
-      const int vcol = blockIdx.x * CT + cc;
-      vs[t * CT + cc] = vcol < dv ? v[(size_t)(row0 + t0 + t) * ld + (size_t)h * dv + vcol] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kScanLoadsV; ++i) {
+      const int idx = tid + i * nthr;
+      if (idx < CH * CT) vs[idx] = pv[i];
     }
     __syncthreads();
+    if (t0 + CH < len) fetch(t0 + CH);
     for (int t = 0; t < nt; ++t) {
       const float vv = vs[t * CT + c];
       const float* qt = qs + t * dkp + r0;
@@ -279,7 +308,8 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
       for (int ss = 1; ss < NS; ++ss) o += part[(t * NS + ss) * CT + cc];
       out[(size_t)(row0 + t0 + t) * ((size_t)H * dv) + (size_t)h * dv + ocol] = o;
     }
-    __syncthreads();
+    // (the next chunk's LDS stores touch qs / ks / ds / vs only; `part` is rewritten after the
+    // barrier that follows them)
   }
   if (col < dv) {
 #pragma unroll
@@ -348,83 +378,213 @@ __global__ void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __res
 
 // Position i sees the tokens j with 0 <= i - j < window and the pooled blocks b with
 // b*pool + pool - 1 <= i - window.  Weight of a key: sigmoid(q.k * scale + head_bias[h]); the
-// weighted values are summed, not normalised.  One workgroup per (row, query head).
+// weighted values are summed, not normalised.  One workgroup per (row, kv head, group of up to
+// kAttnHeads query heads of that kv head): a key or value row is read once for all of them.
+// Phase 1, a thread per key of a 256-key tile: its scores against the query heads (q in LDS).
+// Phase 2, a wave per key, lanes over value columns: the weighted sum.  Keys are taken in the
+// order pooled blocks, then tokens, whatever the batch: a row's bits depend on its position only.
 constexpr int kAttnTile = 256;
-constexpr int kAttnCols = 4;  // value columns per lane: vdim <= 256
-template <typename T>
+constexpr int kAttnBatch = 8;   // value rows a wave has in flight
+constexpr int kAttnLoads = 16;  // 16-byte pieces of a key row a thread has in flight
+constexpr int kAttnSplitRows = 64;  // batches of at most this many rows may split their keys over workgroups
+
+template <typename T> struct Piece;   // a 16-byte piece of a row as floats
+template <> struct Piece<bf16_t> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& raw, float* f) {
+    const bf16x8 v = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+  }
+};
+template <> struct Piece<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void unpack(const u32x4& raw, float* f) {
+    const f32x4 v = __builtin_bit_cast(f32x4, raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = v[i];
+  }
+};
+
+// s[hq] += sum_c qs[hq][c] * k[c], channels in ascending order.  vec: the row is 16-byte aligned
+// and dk a multiple of 8; then up to kAttnLoads pieces of the row are asked for before the first
+// is used.
+template <typename KT, int NH>
+__device__ __forceinline__ void score_key(const KT* __restrict__ kr, const float* __restrict__ qs, int dk, int nh,
+                                          bool vec, float* s) {
+  constexpr int E = Piece<KT>::E;
+  int c = 0;
+  if (vec) {
+    for (; c < dk; c += kAttnLoads * E) {
+      u32x4 raw[kAttnLoads];
+#pragma unroll
+      for (int i = 0; i < kAttnLoads; ++i)
+        if (c + i * E < dk) raw[i] = *reinterpret_cast<const u32x4*>(kr + c + i * E);
+#pragma unroll
+      for (int i = 0; i < kAttnLoads; ++i) {
+        if (c + i * E < dk) {
+          float kf[E];
+          Piece<KT>::unpack(raw[i], kf);
+#pragma unroll
+          for (int hq = 0; hq < NH; ++hq) {
+            if (hq < nh) {
+#pragma unroll
+              for (int e = 0; e < E; ++e) s[hq] = fmaf(qs[hq * dk + c + i * E + e], kf[e], s[hq]);
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
+  for (; c < dk; ++c) {
+    const float kf = ld_f(kr + c);
+#pragma unroll
+    for (int hq = 0; hq < NH; ++hq)
+      if (hq < nh) s[hq] = fmaf(qs[hq * dk + c], kf, s[hq]);
+  }
+}
+
+// NH: query heads per workgroup (of one kv head), NC: value columns per lane (vdim <= 64 * NC).
+// n_splits > 1: workgroup (.., .., z) takes the keys of tile z / n_hgroups only and writes its sum
+// to out + split * split_stride (sum_splits_kernel adds the splits in order).
+template <typename T, int NH, int NC>
 __global__ __launch_bounds__(256) void window_pool_attn_kernel(
     const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const float* __restrict__ pk_cache, const float* __restrict__ pv_cache,
     const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
     const int32_t* __restrict__ block_tables, int max_blocks, int page, int pslots, int H, int G, int dk,
     int dv, int window, int pool, float scale, const float* __restrict__ head_bias,
-    float* __restrict__ out) {
+    float* __restrict__ out, int n_hgroups, int n_splits, size_t split_stride) {
   extern __shared__ float lds[];
   unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [kAttnTile] cache row of the value
-  float* wt = reinterpret_cast<float*>(vat + kAttnTile);                 // [kAttnTile]
-  int* kind = reinterpret_cast<int*>(wt + kAttnTile);                    // [kAttnTile] 1 = pooled
-  float* qs = reinterpret_cast<float*>(kind + kAttnTile);                // [dk]
-  float* red = qs + dk;                                                  // [4][dv]
-  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const int g = h / (H / G);
+  int* kind = reinterpret_cast<int*>(vat + kAttnTile);                   // [kAttnTile] 1 = pooled
+  float* wt = reinterpret_cast<float*>(kind + kAttnTile);                // [NH][kAttnTile]
+  float* qs = wt + NH * kAttnTile;                                       // [nh][dk]
+  float* red = qs + NH * dk;                                             // [4][nh][dv]
+  const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+  const int hgroup = blockIdx.z % n_hgroups, split = blockIdx.z / n_hgroups;
+  const int qh = H / G;
+  const int h0 = g * qh + hgroup * NH;                                   // first query head here
+  const int nh = qh - hgroup * NH < NH ? qh - hgroup * NH : NH;
   const int i = row_pos[r];
   const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
-  for (int c = tid; c < dk; c += 256) qs[c] = q[(size_t)r * ldq + (size_t)h * dk + c];
+  for (int c = tid; c < nh * dk; c += 256) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
   const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
   const int n_blocks = i - window + 1 >= 0 ? (i - window + 1) / pool : 0;
   const int total = n_blocks + (i - t_first + 1);
-  const float bias = head_bias ? head_bias[h] : 0.f;
-  const int wave = tid >> 6, lane = tid & 63;
-  float acc[kAttnCols];
+  const int key_lo = n_splits > 1 ? split * kAttnTile : 0;
+  const int key_hi = n_splits > 1 ? (total < key_lo + kAttnTile ? total : key_lo + kAttnTile) : total;
+  const bool vec_t = dk % 8 == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
+  const bool vec_p = dk % 8 == 0 && (reinterpret_cast<uintptr_t>(pk_cache) & 15) == 0;
+  float bias[NH];
 #pragma unroll
-  for (int m = 0; m < kAttnCols; ++m) acc[m] = 0.f;
+  for (int hq = 0; hq < NH; ++hq) bias[hq] = (head_bias && hq < nh) ? head_bias[h0 + hq] : 0.f;
+  const int wave = tid >> 6, lane = tid & 63;
+  float acc[NH][NC];
+#pragma unroll
+  for (int hq = 0; hq < NH; ++hq)
+#pragma unroll
+    for (int m = 0; m < NC; ++m) acc[hq][m] = 0.f;
   __syncthreads();
-  for (int base = 0; base < total; base += kAttnTile) {
+  for (int base = key_lo; base < key_hi; base += kAttnTile) {
     const int idx = base + tid;
-    if (idx < total) {
-      float s = 0.f;
+    if (idx < key_hi) {
+      float s[NH];
+#pragma unroll
+      for (int hq = 0; hq < NH; ++hq) s[hq] = 0.f;
       if (idx < n_blocks) {
         const int last = idx * pool + pool - 1, lp = last / page;
         const size_t at = ((size_t)tbl[lp] * G + g) * pslots + pooled_slot(idx, lp, page, pool);
-        const float* kr = pk_cache + at * dk;
-        for (int c = 0; c < dk; ++c) s = fmaf(qs[c], kr[c], s);
+        score_key<float, NH>(pk_cache + at * dk, qs, dk, nh, vec_p, s);
         kind[tid] = 1;
         vat[tid] = at;
       } else {
         const int j = t_first + (idx - n_blocks);
         const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
-        const T* kr = k_cache + at * dk;
-        for (int c = 0; c < dk; ++c) s = fmaf(qs[c], ld_f(kr + c), s);
+        score_key<T, NH>(k_cache + at * dk, qs, dk, nh, vec_t, s);
         kind[tid] = 0;
         vat[tid] = at;
       }
-      wt[tid] = sigmoid_f(s * scale + bias);
+#pragma unroll
+      for (int hq = 0; hq < NH; ++hq)
+        if (hq < nh) wt[hq * kAttnTile + tid] = sigmoid_f(s[hq] * scale + bias[hq]);
     }
     __syncthreads();
-    const int n_here = total - base < kAttnTile ? total - base : kAttnTile;
-    for (int kk = wave; kk < n_here; kk += 4) {
-      const float w = wt[kk];
-      const size_t at = vat[kk];
-      if (kind[kk]) {
-        const float* vr = pv_cache + at * dv;
+    const int n_here = key_hi - base < kAttnTile ? key_hi - base : kAttnTile;
+    // a wave takes keys wave, wave + 4, ...; kAttnBatch value rows are asked for before any is used
+    for (int kk0 = wave; kk0 < n_here; kk0 += 4 * kAttnBatch) {
+      float vf[kAttnBatch][NC];
 #pragma unroll
-        for (int m = 0; m < kAttnCols; ++m)
-          if (lane + 64 * m < dv) acc[m] = fmaf(w, vr[lane + 64 * m], acc[m]);
-      } else {
+      for (int u = 0; u < kAttnBatch; ++u) {
+        const int kk = kk0 + 4 * u;
+        const bool on = kk < n_here;
+        const size_t at = on ? vat[kk] : 0;
+        const bool pooled = on && kind[kk];
+        const float* vp = pv_cache + at * dv;
         const T* vr = v_cache + at * dv;
 #pragma unroll
-        for (int m = 0; m < kAttnCols; ++m)
-          if (lane + 64 * m < dv) acc[m] = fmaf(w, ld_f(vr + lane + 64 * m), acc[m]);
+        for (int m = 0; m < NC; ++m) {
+          const bool in = on && lane + 64 * m < dv;
+          vf[u][m] = !in ? 0.f : (pooled ? vp[lane + 64 * m] : ld_f(vr + lane + 64 * m));
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kAttnBatch; ++u) {
+        const int kk = kk0 + 4 * u;
+        if (kk < n_here) {
+#pragma unroll
+          for (int hq = 0; hq < NH; ++hq) {
+            if (hq < nh) {
+              const float w = wt[hq * kAttnTile + kk];
+#pragma unroll
+              for (int m = 0; m < NC; ++m) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
+            }
+          }
+        }
       }
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int m = 0; m < kAttnCols; ++m)
-    if (lane + 64 * m < dv) red[wave * dv + lane + 64 * m] = acc[m];
+  for (int hq = 0; hq < NH; ++hq)
+    if (hq < nh)
+#pragma unroll
+      for (int m = 0; m < NC; ++m)
+        if (lane + 64 * m < dv) red[((size_t)wave * nh + hq) * dv + lane + 64 * m] = acc[hq][m];
   __syncthreads();
-  for (int c = tid; c < dv; c += 256)
-    out[(size_t)r * H * dv + (size_t)h * dv + c] = ((red[c] + red[dv + c]) + red[2 * dv + c]) + red[3 * dv + c];
+  float* dst = out + (n_splits > 1 ? (size_t)split * split_stride : 0);
+  for (int c = tid; c < nh * dv; c += 256) {
+    const size_t step = (size_t)nh * dv;
+    dst[(size_t)r * H * dv + (size_t)h0 * dv + c] = ((red[c] + red[step + c]) + red[2 * step + c]) + red[3 * step + c];
+  }
+}
+
+// out[i] = part[0][i] + part[1][i] + ... in split order
+__global__ void sum_splits_kernel(const float* __restrict__ part, size_t split_stride, int n_splits,
+                                  float* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float sum = part[i];
+  for (int sp = 1; sp < n_splits; ++sp) sum += part[(size_t)sp * split_stride + i];
+  out[i] = sum;
+}
+
+template <typename T, int NH>
+void launch_attn_nc(dim3 grid, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq, const void* kc,
+                    const void* vc, const float* pk, const float* pv, const int32_t* row_pos,
+                    const int32_t* row_slot, const int32_t* bt, int max_blocks, int page, int pslots, int H, int G,
+                    int dk, int dv, int window, int pool, float scale, const float* head_bias, float* out,
+                    int n_hgroups, int n_splits, size_t split_stride) {
+#define SD_ATTN_GO(NC)                                                                                           \
+  window_pool_attn_kernel<T, NH, NC><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, pk, pv, row_pos, \
+                                                             row_slot, bt, max_blocks, page, pslots, H, G, dk, dv, \
+                                                             window, pool, scale, head_bias, out, n_hgroups,       \
+                                                             n_splits, split_stride)
+  if (nc == 1) SD_ATTN_GO(1);
+  else if (nc == 2) SD_ATTN_GO(2);
+  else SD_ATTN_GO(4);
+#undef SD_ATTN_GO
 }
 
 // x += sigmoid(z1 + c1) * a + sigmoid(z2 + c2) * b   (b == nullptr: one sublayer; c1, c2 may be null)
@@ -532,8 +692,11 @@ extern "C" int sd_decay_scan(const float* q, const float* k, const float* v, int
   if (CT > dv) CT = dv;
   if (CT > 64) CT = 64;
   const int tiles = (dv + CT - 1) / CT;
-  const int CH = dk > 128 ? 8 : 16;
   const int dkp = NS * kStrip;
+  int CH = kScanLoads * (CT * NS) / dkp;   // a chunk's q / k elements fit kScanLoads per thread
+  if (CH > 16) CH = 16;
+  SD_REQUIRE(CH >= 1 && CH * CT <= kScanLoadsV * CT * NS, SD_ERR_UNSUPPORTED,
+             "sd_decay_scan: key size %d with value size %d leaves no chunk", dk, dv);
   const size_t lds = sizeof(float) * ((size_t)(per_channel ? 3 : 2) * CH * dkp + (size_t)CH * CT + (size_t)CH * NS * CT);
   dim3 grid(tiles, H, n_entries);
   hipStream_t st = (hipStream_t)stream;
@@ -564,39 +727,73 @@ extern "C" int sd_pooled_slots_per_page(int page, int pool) {
   return page / pool + 2;
 }
 
+extern "C" size_t sd_window_pool_attention_scratch_bytes(int n_rows, int H, int dv, int window, int pool,
+                                                        int max_ctx) {
+  if (n_rows < 1 || n_rows > kAttnSplitRows || pool < 1) return 0;
+  const int max_keys = window + max_ctx / pool + 1;
+  const int splits = (max_keys + kAttnTile - 1) / kAttnTile;
+  return splits > 1 ? (size_t)splits * n_rows * H * dv * sizeof(float) : 0;
+}
+
 extern "C" int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
                                         int cache_f32, float* pk_cache, float* pv_cache,
                                         const int32_t* row_pos, const int32_t* row_slot,
                                         const int32_t* block_tables, int max_blocks, int page, int n_rows,
                                         int H, int G, int dk, int dv, int window, int pool, float scale,
-                                        const float* head_bias, float* out, sd_stream_t stream) {
+                                        const float* head_bias, float* out, void* scratch, size_t scratch_bytes,
+                                        sd_stream_t stream) {
   SD_REQUIRE(q && k_cache && v_cache && pk_cache && pv_cache && row_pos && row_slot && block_tables && out,
              SD_ERR_INVALID, "sd_window_pool_attention: null argument");
   SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && pool >= 1 && page >= 1,
              SD_ERR_INVALID, "sd_window_pool_attention: bad shape");
-  SD_REQUIRE(dv >= 1 && dv <= 64 * kAttnCols, SD_ERR_UNSUPPORTED,
-             "sd_window_pool_attention: value size %d outside 1..%d", dv, 64 * kAttnCols);
+  SD_REQUIRE(dv >= 1 && dv <= 256, SD_ERR_UNSUPPORTED, "sd_window_pool_attention: value size %d outside 1..256", dv);
   const int pslots = sd_pooled_slots_per_page(page, pool);
   hipStream_t st = (hipStream_t)stream;
   dim3 gp(n_rows, G);
-  dim3 ga(n_rows, H);
-  const size_t lds = sizeof(float) * (size_t)(dk + kAttnTile * 2 + 4 * dv) + sizeof(unsigned long long) * kAttnTile + 16;
-  if (cache_f32) {
+  const int qh = H / G;
+  const int NH = qh <= 1 ? 1 : (qh <= 2 ? 2 : (qh <= 4 ? 4 : 8));
+  const int nh = qh < NH ? qh : NH;
+  const int n_hgroups = (qh + NH - 1) / NH;
+  const int nc = dv <= 64 ? 1 : (dv <= 128 ? 2 : 4);
+  // Few rows: the keys of a row are cut into tiles that run as workgroups of their own.
+  const size_t need = sd_window_pool_attention_scratch_bytes(n_rows, H, dv, window, pool, max_blocks * page);
+  const bool split = need > 0 && scratch && scratch_bytes >= need;
+  const int n_splits = split ? (int)(need / ((size_t)n_rows * H * dv * sizeof(float))) : 1;
+  const size_t split_stride = (size_t)n_rows * H * dv;
+  dim3 ga(n_rows, G, n_hgroups * n_splits);
+  const size_t lds = sizeof(unsigned long long) * kAttnTile + sizeof(int) * kAttnTile +
+                     sizeof(float) * ((size_t)NH * kAttnTile + (size_t)NH * dk + (size_t)4 * nh * dv);
+  SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_pool_attention: dim %d / vdim %d need %zu bytes of LDS",
+             dk, dv, lds);
+  float* dst = split ? (float*)scratch : out;
+  if (cache_f32)
     pool_blocks_kernel<float><<<gp, 64, 0, st>>>((const float*)k_cache, (const float*)v_cache, pk_cache, pv_cache,
                                                  row_pos, row_slot, block_tables, max_blocks, page, pslots, G, dk, dv, pool);
-    SD_CHECK_LAUNCH("sd_window_pool_attention (pool)");
-    window_pool_attn_kernel<float><<<ga, 256, lds, st>>>(q, ldq, (const float*)k_cache, (const float*)v_cache, pk_cache,
-                                                         pv_cache, row_pos, row_slot, block_tables, max_blocks, page,
-                                                         pslots, H, G, dk, dv, window, pool, scale, head_bias, out);
-  } else {
+  else
     pool_blocks_kernel<bf16_t><<<gp, 64, 0, st>>>((const bf16_t*)k_cache, (const bf16_t*)v_cache, pk_cache, pv_cache,
                                                   row_pos, row_slot, block_tables, max_blocks, page, pslots, G, dk, dv, pool);
-    SD_CHECK_LAUNCH("sd_window_pool_attention (pool)");
-    window_pool_attn_kernel<bf16_t><<<ga, 256, lds, st>>>(q, ldq, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pk_cache,
-                                                          pv_cache, row_pos, row_slot, block_tables, max_blocks, page,
-                                                          pslots, H, G, dk, dv, window, pool, scale, head_bias, out);
-  }
+  SD_CHECK_LAUNCH("sd_window_pool_attention (pool)");
+#define SD_ATTN_NH(T, N)                                                                                          \
+  launch_attn_nc<T, N>(ga, lds, st, nc, q, ldq, k_cache, v_cache, pk_cache, pv_cache, row_pos, row_slot, block_tables, \
+                       max_blocks, page, pslots, H, G, dk, dv, window, pool, scale, head_bias, dst, n_hgroups,     \
+                       n_splits, split_stride)
+#define SD_ATTN_T(T)                  \
+  do {                                \
+    if (NH == 1) SD_ATTN_NH(T, 1);    \
+    else if (NH == 2) SD_ATTN_NH(T, 2); \
+    else if (NH == 4) SD_ATTN_NH(T, 4); \
+    else SD_ATTN_NH(T, 8);            \
+  } while (0)
+  if (cache_f32) SD_ATTN_T(float);
+  else SD_ATTN_T(bf16_t);
+#undef SD_ATTN_T
+#undef SD_ATTN_NH
   SD_CHECK_LAUNCH("sd_window_pool_attention");
+  if (split) {
+    const size_t n = split_stride;
+    sum_splits_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const float*)scratch, split_stride, n_splits, out, n);
+    SD_CHECK_LAUNCH("sd_window_pool_attention (sum)");
+  }
   return SD_OK;
 }
 
@@ -646,11 +843,11 @@ InCols in_cols(const sd_seq_layer& l, int W) {
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr int kWideRows = 256;  // rows one call of the many-row linear family takes
 struct SeqWs {
-  size_t x, h, proj, dec, o, y, mix, ffo, hout, hb, yb, actb, houtb, wide, wide_bytes, total;
+  size_t x, h, proj, dec, o, y, mix, ffo, hout, hb, yb, actb, houtb, wide, wide_bytes, attn, attn_bytes, total;
 };
-SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
+SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
   const int W = m.d.width;
-  size_t proj = 0, hk = 0, hv = 0, ff = 0, wide = 0;
+  size_t proj = 0, hk = 0, hv = 0, ff = 0, wide = 0, attn = 0;
   const int wr = rows < kWideRows ? rows : kWideRows;
   auto need = [&](const void* tiled, int M, int N, int K) {
     if (!tiled || M <= 16) return;
@@ -667,6 +864,10 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
     need(l.w_in_tiled, wr, (int)t, W);
     need(l.w_o_tiled, wr, W, l.heads * l.vdim);
     need(l.w_down_tiled, wr, W, l.ff);
+    if (l.kind == SD_MIX_WINDOW_POOL) {
+      const size_t n = sd_window_pool_attention_scratch_bytes(rows, l.heads, l.vdim, l.window, l.pool, max_ctx);
+      attn = n > attn ? n : attn;
+    }
   }
   const int no = n_out > 0 ? n_out : 1;
   need(m.d.head_tiled, no < kWideRows ? no : kWideRows, m.d.vocab, W);
@@ -689,6 +890,8 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out) {
   w.houtb = off; off += al((size_t)no * W * 2);
   w.wide_bytes = wide;
   w.wide = off; off += al(wide ? wide : 16);
+  w.attn_bytes = attn;
+  w.attn = off; off += al(attn ? attn : 16);
   w.total = off;
   return w;
 }
@@ -751,9 +954,12 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
 
 extern "C" void sd_seq_model_destroy(sd_seq_model* m) { delete m; }
 
-extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out) {
+extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_rows, int max_out, int max_ctx) {
   if (!m || max_rows < 1) return 0;
-  return plan_seq(*m, max_rows, max_out).total;
+  // (the split scratch of the window layers exists for small batches only: take the larger plan)
+  const size_t a = plan_seq(*m, max_rows, max_out, max_ctx).total;
+  const size_t b = plan_seq(*m, max_rows < kAttnSplitRows ? max_rows : kAttnSplitRows, max_out, max_ctx).total;
+  return a > b ? a : b;
 }
 
 #define SQ_TRY(expr)                \
@@ -769,7 +975,7 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
              SD_ERR_INVALID, "sd_seq_model_forward: empty batch or null array");
   SD_REQUIRE(b->n_out >= 0 && (b->n_out == 0 || (b->out_rows && b->logits)), SD_ERR_INVALID,
              "sd_seq_model_forward: wanted rows need out_rows and logits");
-  const SeqWs w = plan_seq(*m, b->n_rows, b->n_out);
+  const SeqWs w = plan_seq(*m, b->n_rows, b->n_out, b->max_blocks * b->page);
   SD_REQUIRE(workspace_bytes >= w.total, SD_ERR_WORKSPACE, "sd_seq_model_forward: workspace %zu < %zu bytes",
              workspace_bytes, w.total);
   SD_REQUIRE(sd_aligned16(workspace), SD_ERR_INVALID, "sd_seq_model_forward: workspace unaligned");
@@ -813,7 +1019,8 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
                           l.k_cache, l.v_cache, f32, b->block_tables, b->max_blocks, b->page, stream));
       SQ_TRY(sd_window_pool_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, l.pk_cache, l.pv_cache,
                                       b->row_pos, b->row_slot, b->block_tables, b->max_blocks, b->page, R, H, G,
-                                      dk, dv, l.window, l.pool, l.score_scale, l.head_bias, o, stream));
+                                      dk, dv, l.window, l.pool, l.score_scale, l.head_bias, o, base + w.attn,
+                                      w.attn_bytes, stream));
       SQ_TRY(sd_head_post(o, proj + c.g, ld, nullptr, f32, 0, d.norm_eps, 1, y, y_b, R, H, dv, rnd, stream));
     } else {
       SQ_TRY(sd_head_prep(proj + c.q, proj + c.k, nullptr, ld, b->row_pos, b->row_slot, R, H, H, dk, dv,

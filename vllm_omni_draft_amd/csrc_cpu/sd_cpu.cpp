@@ -1478,9 +1478,10 @@ extern "C" int sd_decay_scan(const float*, const float*, const float*, int64_t, 
 extern "C" int sd_head_post(const float*, const float*, int64_t, const void*, int, int, float, int, float*, void*,
                             int, int, int, int, sd_stream_t) { UNSUPPORTED("sd_head_post"); }
 extern "C" int sd_pooled_slots_per_page(int page, int pool) { return page < 1 || pool < 1 ? 0 : page / pool + 2; }
+extern "C" size_t sd_window_pool_attention_scratch_bytes(int, int, int, int, int, int) { return 0; }
 extern "C" int sd_window_pool_attention(const float*, int64_t, const void*, const void*, int, float*, float*,
                                         const int32_t*, const int32_t*, const int32_t*, int, int, int, int, int,
-                                        int, int, int, int, float, const float*, float*, sd_stream_t) {
+                                        int, int, int, int, float, const float*, float*, void*, size_t, sd_stream_t) {
   UNSUPPORTED("sd_window_pool_attention");
 }
 extern "C" int sd_gated_residual(float*, const float*, const float*, int64_t, const float*, const float*,
@@ -1493,7 +1494,7 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc*) {
   return nullptr;
 }
 extern "C" void sd_seq_model_destroy(sd_seq_model*) {}
-extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model*, int, int) { return 0; }
+extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model*, int, int, int) { return 0; }
 extern "C" int sd_seq_model_forward(sd_seq_model*, const sd_seq_batch*, void*, size_t, sd_stream_t) {
   UNSUPPORTED("sd_seq_model_forward");
 }

@@ -267,7 +267,8 @@ class SeqModel:
         if self.workspace is not None and rows <= self._ws_rows and n_out <= self._ws_out:
             return
         self._ws_rows, self._ws_out = max(rows, self._ws_rows), max(n_out, self._ws_out, 1)
-        n = _lib.load().sd_seq_model_workspace_bytes(self._handle, self._ws_rows, self._ws_out)
+        n = _lib.load().sd_seq_model_workspace_bytes(self._handle, self._ws_rows, self._ws_out,
+                                                     self.cache.max_blocks_per_seq * self.cache.page)
         self.workspace = torch.empty(int(n), dtype=torch.uint8, device=self.weights.embed.device)
 
     def forward(self, n_rows: int, n_entries: int, tokens, row_pos, row_slot, entries, n_out: int,

@@ -1135,15 +1135,20 @@ def head_post(o, g, H, dv, *, norm_w=None, unit_norm=False, eps=1e-5, gate="silu
 
 
 def window_pool_attention(q, k_cache, v_cache, pk_cache, pv_cache, row_pos, row_slot, block_tables, H, G,
-                          dk, dv, window, pool, scale, head_bias=None) -> torch.Tensor:
+                          dk, dv, window, pool, scale, head_bias=None, split=True) -> torch.Tensor:
     """q f32 [rows, H*dk] (prepared); caches as kv_cache.SeqCache lays them out; returns f32
     [rows, H*dv].  Also fills the pooled entries of blocks that these rows complete."""
     _f32(q, "q")
     out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
-    _lib.check(_lib.load().sd_window_pool_attention(
+    lib = _lib.load()
+    n = int(lib.sd_window_pool_attention_scratch_bytes(q.shape[0], H, dv, window, pool,
+                                                       block_tables.shape[1] * PAGE)) if split else 0
+    scratch = torch.empty(n, dtype=torch.uint8, device=q.device) if n else None
+    _lib.check(lib.sd_window_pool_attention(
         _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(pk_cache),
         _p(pv_cache), _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0],
-        H, G, dk, dv, window, pool, float(scale), _p(head_bias), _p(out), _stream()), "sd_window_pool_attention")
+        H, G, dk, dv, window, pool, float(scale), _p(head_bias), _p(out), _p(scratch), n, _stream()),
+        "sd_window_pool_attention")
     return out
 
 
