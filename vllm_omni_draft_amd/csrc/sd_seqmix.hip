@@ -217,6 +217,7 @@ __global__ void sigmoid_power_kernel(const float* __restrict__ z, int64_t ldz, f
 constexpr int kStrip = 16;
 constexpr int kScanLoads = 8;    // q / k / decay elements a thread stages per chunk, at most
 constexpr int kScanLoadsV = 16;  // value elements
+constexpr int kScanChunk = 16;   // tokens per chunk, at most
 template <bool PER_CHANNEL>
 __global__ __launch_bounds__(256) void decay_scan_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, int64_t ld,
@@ -252,18 +253,26 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
       const int idx = tid + i * nthr;
       const int t = idx / dkp, ch = idx % dkp;
       const bool in = idx < nt * dkp && ch < dk;
-      const size_t at = (size_t)(row0 + t0 + (in ? t : 0)) * ld + (size_t)h * dk + (in ? ch : 0);
-      pq[i] = in ? q[at] : 0.f;
-      pk[i] = in ? k[at] : 0.f;
-      if (PER_CHANNEL)
-        pd[i] = in ? decay[(size_t)(row0 + t0 + t) * ((size_t)H * dk) + (size_t)h * dk + ch] : 0.f;
+      // (every load is issued, on an address clamped into the chunk: a guarded load would become
+      // a branch whose join waits for the loads in flight)
+      const int tc = t < nt ? t : nt - 1, cc = ch < dk ? ch : dk - 1;
+      const size_t at = (size_t)(row0 + t0 + tc) * ld + (size_t)h * dk + cc;
+      const float lq = q[at], lk = k[at];
+      pq[i] = in ? lq : 0.f;
+      pk[i] = in ? lk : 0.f;
+      if (PER_CHANNEL) {
+        const float ldc = decay[(size_t)(row0 + t0 + tc) * ((size_t)H * dk) + (size_t)h * dk + cc];
+        pd[i] = in ? ldc : 0.f;
+      }
     }
 #pragma unroll
     for (int i = 0; i < kScanLoadsV; ++i) {
       const int idx = tid + i * nthr;
       const int t = idx / CT, vcol = blockIdx.x * CT + idx % CT;
       const bool in = idx < nt * CT && vcol < dv;
-      pv[i] = in ? v[(size_t)(row0 + t0 + t) * ld + (size_t)h * dv + vcol] : 0.f;
+      const int tc = t < nt ? t : nt - 1, vc2 = vcol < dv ? vcol : dv - 1;
+      const float lv = v[(size_t)(row0 + t0 + tc) * ld + (size_t)h * dv + vc2];
+      pv[i] = in ? lv : 0.f;
     }
   };
   fetch(0);
@@ -418,8 +427,10 @@ __device__ __forceinline__ void score_key(const KT* __restrict__ kr, const float
     for (; c < dk; c += kAttnLoads * E) {
       u32x4 raw[kAttnLoads];
 #pragma unroll
-      for (int i = 0; i < kAttnLoads; ++i)
-        if (c + i * E < dk) raw[i] = *reinterpret_cast<const u32x4*>(kr + c + i * E);
+      for (int i = 0; i < kAttnLoads; ++i) {   // unguarded, on an address clamped into the row
+        const int ci = c + i * E < dk ? c + i * E : dk - E;
+        raw[i] = *reinterpret_cast<const u32x4*>(kr + ci);
+      }
 #pragma unroll
       for (int i = 0; i < kAttnLoads; ++i) {
         if (c + i * E < dk) {
@@ -512,38 +523,39 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(
     }
     __syncthreads();
     const int n_here = key_hi - base < kAttnTile ? key_hi - base : kAttnTile;
-    // a wave takes keys wave, wave + 4, ...; kAttnBatch value rows are asked for before any is used
-    for (int kk0 = wave; kk0 < n_here; kk0 += 4 * kAttnBatch) {
-      float vf[kAttnBatch][NC];
+    // A wave takes every fourth key; kAttnBatch value rows are asked for before any is used.  The
+    // tile's pooled keys come first, then its tokens: each loop reads one element type, with
+    // unguarded loads on clamped addresses.
+    const int nb_here = n_blocks - base < 0 ? 0 : (n_blocks - base < n_here ? n_blocks - base : n_here);
+    auto sweep = [&](int lo, int hi, auto load_row) {
+      for (int kk0 = lo + wave; kk0 < hi; kk0 += 4 * kAttnBatch) {
+        float vf[kAttnBatch][NC];
 #pragma unroll
-      for (int u = 0; u < kAttnBatch; ++u) {
-        const int kk = kk0 + 4 * u;
-        const bool on = kk < n_here;
-        const size_t at = on ? vat[kk] : 0;
-        const bool pooled = on && kind[kk];
-        const float* vp = pv_cache + at * dv;
-        const T* vr = v_cache + at * dv;
+        for (int u = 0; u < kAttnBatch; ++u) {
+          const int kk = kk0 + 4 * u < hi ? kk0 + 4 * u : hi - 1;
+          const size_t at = vat[kk];
 #pragma unroll
-        for (int m = 0; m < NC; ++m) {
-          const bool in = on && lane + 64 * m < dv;
-          vf[u][m] = !in ? 0.f : (pooled ? vp[lane + 64 * m] : ld_f(vr + lane + 64 * m));
+          for (int m = 0; m < NC; ++m) vf[u][m] = load_row(at, lane + 64 * m < dv ? lane + 64 * m : dv - 1);
         }
-      }
 #pragma unroll
-      for (int u = 0; u < kAttnBatch; ++u) {
-        const int kk = kk0 + 4 * u;
-        if (kk < n_here) {
+        for (int u = 0; u < kAttnBatch; ++u) {
+          const int kk = kk0 + 4 * u;
+          if (kk < hi) {
 #pragma unroll
-          for (int hq = 0; hq < NH; ++hq) {
-            if (hq < nh) {
-              const float w = wt[hq * kAttnTile + kk];
+            for (int hq = 0; hq < NH; ++hq) {
+              if (hq < nh) {
+                const float w = wt[hq * kAttnTile + kk];
 #pragma unroll
-              for (int m = 0; m < NC; ++m) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
+                for (int m = 0; m < NC; ++m)
+                  if (lane + 64 * m < dv) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
+              }
             }
           }
         }
       }
-    }
+    };
+    sweep(0, nb_here, [&](size_t at, int col) { return pv_cache[at * dv + col]; });
+    sweep(nb_here, n_here, [&](size_t at, int col) { return ld_f(v_cache + at * dv + col); });
     __syncthreads();
   }
 #pragma unroll
@@ -688,18 +700,18 @@ extern "C" int sd_decay_scan(const float* q, const float* k, const float* v, int
              SD_ERR_INVALID, "sd_decay_scan: bad argument");
   SD_REQUIRE(dk >= 1 && dk <= 256, SD_ERR_UNSUPPORTED, "sd_decay_scan: key size %d outside 1..256", dk);
   const int NS = (dk + kStrip - 1) / kStrip;
+  hipStream_t st = (hipStream_t)stream;
   int CT = 256 / NS;
   if (CT > dv) CT = dv;
   if (CT > 64) CT = 64;
   const int tiles = (dv + CT - 1) / CT;
   const int dkp = NS * kStrip;
   int CH = kScanLoads * (CT * NS) / dkp;   // a chunk's q / k elements fit kScanLoads per thread
-  if (CH > 16) CH = 16;
+  if (CH > kScanChunk) CH = kScanChunk;
   SD_REQUIRE(CH >= 1 && CH * CT <= kScanLoadsV * CT * NS, SD_ERR_UNSUPPORTED,
              "sd_decay_scan: key size %d with value size %d leaves no chunk", dk, dv);
   const size_t lds = sizeof(float) * ((size_t)(per_channel ? 3 : 2) * CH * dkp + (size_t)CH * CT + (size_t)CH * NS * CT);
   dim3 grid(tiles, H, n_entries);
-  hipStream_t st = (hipStream_t)stream;
   if (per_channel)
     decay_scan_kernel<true><<<grid, CT * NS, lds, st>>>(q, k, v, ld, decay, state, entries, out, H, dk, dv, CT, NS, CH);
   else
