@@ -4,10 +4,14 @@
     python examples/generate.py --target-dir /models/Llama-3-8B --draft-dir /models/Llama-3.2-1B \\
                                 --prompt-ids 128000 9906 1917
 
+    python examples/generate.py --model-dir /models/some-puguzen --dtype float32 --prompt-ids 5 17 3
+
 With --target-dir / --draft-dir the models are read from local Hugging Face checkpoints
 (config.json + *.safetensors); without them, seeded random weights of the named presets stand in
-(the output is then meaningless, the timing is not).  Tokenisation is the caller's: prompts are
-token ids.
+(the output is then meaningless, the timing is not).  --model-dir serves a layer-list model
+(recurrent / windowed layers; config.json names its "architecture") without speculation through
+the same scheduler, in bfloat16 or float32.
+Tokenisation is the caller's: prompts are token ids.
 """
 import argparse
 import os
@@ -30,8 +34,40 @@ def load(model_dir, preset, vocab=None, seed=0, fp8=False):
     return weights.random_init(cfg, seed=seed, fp8=fp8)
 
 
+def serve_single(args):
+    """--model-dir: one model, chosen by its config.json, through the scheduler."""
+    from vllm_omni_draft_amd.config import SeqModelConfig, load_model_config
+    cfg = load_model_config(args.model_dir)
+    dtype = torch.float32 if args.dtype == "float32" else torch.bfloat16
+    if not isinstance(cfg, SeqModelConfig):
+        raise SystemExit("--model-dir serves layer-list models; give a Hugging Face decoder as --target-dir "
+                         "with its --draft-dir")
+    from vllm_omni_draft_amd.seq_engine import SeqWorker, SeqWorkerConfig
+    w = weights.seq_from_safetensors_dir(cfg, args.model_dir, "cuda", dtype)
+    worker = SeqWorker(SeqWorkerConfig(w, max_num_seqs=args.max_num_seqs, max_model_len=2048))
+    worker.init_device()
+    worker.load_model()
+    sched = SpecDecodeScheduler.for_worker(worker)
+    g = torch.Generator().manual_seed(0)
+    prompts = [list(args.prompt_ids)] if args.prompt_ids else \
+        [torch.randint(0, cfg.vocab, (n,), generator=g).tolist() for n in (12, 200, 57, 1000)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reqs = sched.generate(prompts, max_tokens=args.max_tokens)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for r in reqs:
+        print(f"{r.request_id}: prompt of {len(r.prompt_token_ids)} tokens -> {r.output_token_ids[:12]}"
+              f"{' ...' if len(r.output_token_ids) > 12 else ''} ({r.finish_reason})")
+    n = sum(len(r.output_token_ids) for r in reqs)
+    print(f"{n} tokens in {dt * 1e3:.1f} ms ({n / dt:.0f} tokens/s, prefill included)")
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--model-dir", help="serve a layer-list model (config.json \"architecture\"), no draft")
+    ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16",
+                    help="--model-dir: serving dtype")
     ap.add_argument("--target-dir")
     ap.add_argument("--draft-dir")
     ap.add_argument("--target", default="llama-3-8b", help="preset name when no --target-dir is given")
@@ -42,6 +78,9 @@ def main():
     ap.add_argument("--fp8", action="store_true", help="quantise both models' matrices to fp8 at load")
     ap.add_argument("--prompt-ids", type=int, nargs="*", help="one prompt as token ids (default: four random ones)")
     args = ap.parse_args()
+    if args.model_dir:
+        serve_single(args)
+        return
 
     target = load(args.target_dir, args.target, fp8=args.fp8)
     draft = load(args.draft_dir, args.draft, vocab=target.cfg.vocab, seed=1, fp8=args.fp8)

@@ -3,8 +3,6 @@ every mechanism alone through its entry point, then whole models through the eng
 whole, token by token, in portions, in mixed batches, over reused slots and pages) and through
 the worker and scheduler.  Small random models of several shapes; where random weights would hide
 a fault (one far key among many, a window's edge) the inputs are made so that it shows."""
-import math
-
 import pytest
 import torch
 
@@ -64,9 +62,10 @@ SHAPES = {
                        layer("attention", heads=4, kv_heads=4, dim=16, vdim=8, window=20, pool=32, ff=24)],
                       width=40, vocab=50),
     # widths that are multiples of 32: bfloat16 serving takes the tiled linear kernels everywhere
-    "aligned": model_cfg([layer("gla", heads=4, dim=32, vdim=16, rank=32, ff=160),
+    # (with a stacked input matrix of an odd number of rows, and a vocabulary that is no multiple of 4)
+    "aligned": model_cfg([layer("gla", heads=4, dim=32, vdim=16, rank=5, ff=160),
                           layer("attention", heads=4, kv_heads=2, dim=32, vdim=24, window=12, pool=2, ff=64),
-                          layer("retention", heads=2, dim=16, vdim=48, ff=0)], width=128, vocab=176),
+                          layer("retention", heads=2, dim=16, vdim=48, ff=0)], width=128, vocab=178),
     "wide_heads": model_cfg([layer("gla", heads=2, dim=136, vdim=80, rank=5),
                              layer("attention", heads=2, kv_heads=1, dim=72, vdim=136, window=33, pool=3)],
                             width=48, vocab=64),

@@ -469,8 +469,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(
     float* __restrict__ out, int n_hgroups, int n_splits, size_t split_stride) {
   extern __shared__ float lds[];
   unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [kAttnTile] cache row of the value
-  int* kind = reinterpret_cast<int*>(vat + kAttnTile);                   // [kAttnTile] 1 = pooled
-  float* wt = reinterpret_cast<float*>(kind + kAttnTile);                // [NH][kAttnTile]
+  float* wt = reinterpret_cast<float*>(vat + kAttnTile);                 // [NH][kAttnTile]
   float* qs = wt + NH * kAttnTile;                                       // [nh][dk]
   float* red = qs + NH * dk;                                             // [4][nh][dv]
   const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
@@ -508,13 +507,11 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(
         const int last = idx * pool + pool - 1, lp = last / page;
         const size_t at = ((size_t)tbl[lp] * G + g) * pslots + pooled_slot(idx, lp, page, pool);
         score_key<float, NH>(pk_cache + at * dk, qs, dk, nh, vec_p, s);
-        kind[tid] = 1;
         vat[tid] = at;
       } else {
         const int j = t_first + (idx - n_blocks);
         const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
         score_key<T, NH>(k_cache + at * dk, qs, dk, nh, vec_t, s);
-        kind[tid] = 0;
         vat[tid] = at;
       }
 #pragma unroll
@@ -773,7 +770,7 @@ extern "C" int sd_window_pool_attention(const float* q, int64_t ldq, const void*
   const int n_splits = split ? (int)(need / ((size_t)n_rows * H * dv * sizeof(float))) : 1;
   const size_t split_stride = (size_t)n_rows * H * dv;
   dim3 ga(n_rows, G, n_hgroups * n_splits);
-  const size_t lds = sizeof(unsigned long long) * kAttnTile + sizeof(int) * kAttnTile +
+  const size_t lds = sizeof(unsigned long long) * kAttnTile +
                      sizeof(float) * ((size_t)NH * kAttnTile + (size_t)NH * dk + (size_t)4 * nh * dv);
   SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_pool_attention: dim %d / vdim %d need %zu bytes of LDS",
              dk, dv, lds);
