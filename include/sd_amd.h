@@ -1099,6 +1099,12 @@ int sd_window_pool_attention(const float* q, int64_t ldq, const void* k_cache, c
 int sd_gated_residual(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
                       const float* c2, const float* a, const float* b, int n_rows, int W,
                       sd_stream_t stream);
+/* The same update, then the RMS norm of the updated rows as sd_rmsnorm_rows computes it (the next
+ * layer's input): h, and h_bf16 unless NULL.                                                */
+int sd_gated_residual_norm(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
+                           const float* c2, const float* a, const float* b, int n_rows, int W,
+                           const void* norm_w, int w_f32, float offset, float eps, float* h,
+                           void* h_bf16, sd_stream_t stream);
 /* out_bf16[r, c] = relu(gate[r, c]) * up[r, c]: a gated feed-forward's activation as the bf16
  * operand of sd_linear / sd_linear_wide.                                                   */
 int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, void* out_bf16, int n_rows,

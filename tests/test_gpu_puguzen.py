@@ -212,6 +212,13 @@ def test_gated_residual():
     xd = dev(x)
     ops.gated_residual(xd, dev(z1), dev(a), dev(z2), dev(b), dev(c1), dev(c2))
     assert rel(xd, x + torch.sigmoid(z1 + c1) * a + torch.sigmoid(z2 + c2) * b) < 1e-6
+    # the fused form: the same update, then the next norm
+    w = torch.randn(50, generator=g) * 0.1
+    xd = dev(x)
+    h, h_b = ops.gated_residual_norm(xd, dev(z1), dev(a), dev(w), 1e-5, dev(z2), dev(b), dev(c1), dev(c2))
+    xr = x + torch.sigmoid(z1 + c1) * a + torch.sigmoid(z2 + c2) * b
+    assert rel(xd, xr) < 1e-6 and rel(h, P.offset_rms_norm(xr.double(), w.double(), 1e-5)) < 1e-6
+    assert torch.equal(h_b, h.to(torch.bfloat16))
     act = ops.relu_mul_rows(dev(z1), dev(z2))
     assert torch.equal(act.cpu(), (torch.relu(z1) * z2).to(torch.bfloat16))
 

@@ -222,6 +222,8 @@ SIGNATURES = {
     "sd_window_pool_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                        i32, i32, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]),
     "sd_gated_residual": (i32, [vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, vp]),
+    "sd_gated_residual_norm": (i32, [vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, vp, i32, C.c_float, C.c_float,
+                                     vp, vp, vp]),
     "sd_relu_mul_rows": (i32, [vp, vp, i64, vp, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),

@@ -609,6 +609,33 @@ __global__ void gated_residual_kernel(float* __restrict__ x, const float* __rest
   }
 }
 
+// The same update followed by the next layer's norm of the updated row (one workgroup per row):
+// h = x / sqrt(mean(x^2) + eps) * (offset + w), also as bf16 when h_b is given.
+template <typename T>
+__global__ void gated_residual_norm_kernel(float* __restrict__ x, const float* __restrict__ z1,
+                                           const float* __restrict__ z2, int64_t ldz, const float* __restrict__ c1,
+                                           const float* __restrict__ c2, const float* __restrict__ a,
+                                           const float* __restrict__ b, int W, const T* __restrict__ w, float offset,
+                                           float eps, float* __restrict__ h, bf16_t* __restrict__ h_b, int round) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float add = sigmoid_f(z1[(size_t)r * ldz + c] + (c1 ? c1[c] : 0.f)) * a[(size_t)r * W + c];
+    if (b) add += sigmoid_f(z2[(size_t)r * ldz + c] + (c2 ? c2[c] : 0.f)) * b[(size_t)r * W + c];
+    const float xn = x[(size_t)r * W + c] + add;
+    x[(size_t)r * W + c] = xn;
+    ss = fmaf(xn, xn, ss);
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {   // each thread re-reads what it wrote itself
+    const float v = maybe_round(x[(size_t)r * W + c] * rstd * (offset + ld_f(w + c)), round);
+    h[(size_t)r * W + c] = v;
+    if (h_b) h_b[(size_t)r * W + c] = (bf16_t)v;
+  }
+}
+
 // out[r, c] = bf16(relu(gate[r, c]) * up[r, c]): the gated feed-forward's activation as the bf16
 // operand of the tiled linear kernels
 __global__ void relu_mul_rows_kernel(const float* __restrict__ gate, const float* __restrict__ up, int64_t ld,
@@ -815,6 +842,23 @@ extern "C" int sd_gated_residual(float* x, const float* z1, const float* z2, int
   return SD_OK;
 }
 
+extern "C" int sd_gated_residual_norm(float* x, const float* z1, const float* z2, int64_t ldz, const float* c1,
+                                      const float* c2, const float* a, const float* b, int n_rows, int W,
+                                      const void* norm_w, int w_f32, float offset, float eps, float* h,
+                                      void* h_bf16, sd_stream_t stream) {
+  SD_REQUIRE(x && z1 && a && (!b || z2) && norm_w && h && n_rows >= 1 && W >= 1, SD_ERR_INVALID,
+             "sd_gated_residual_norm: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32)
+    gated_residual_norm_kernel<float><<<n_rows, 256, 0, st>>>(x, z1, z2, ldz, c1, c2, a, b, W, (const float*)norm_w,
+                                                              offset, eps, h, (bf16_t*)h_bf16, 0);
+  else
+    gated_residual_norm_kernel<bf16_t><<<n_rows, 256, 0, st>>>(x, z1, z2, ldz, c1, c2, a, b, W, (const bf16_t*)norm_w,
+                                                               offset, eps, h, (bf16_t*)h_bf16, 1);
+  SD_CHECK_LAUNCH("sd_gated_residual_norm");
+  return SD_OK;
+}
+
 extern "C" int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, void* out_bf16, int n_rows,
                                 int F, sd_stream_t stream) {
   SD_REQUIRE(gate && up && out_bf16 && n_rows >= 1 && F >= 1 && ld >= F, SD_ERR_INVALID,
@@ -1017,7 +1061,10 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
     const InCols c = in_cols(l, W);
     const int64_t ld = c.total;
     const int H = l.heads, G = l.kv_heads, dk = l.dim, dv = l.vdim;
-    SQ_TRY(sd_rmsnorm_rows(x, nullptr, l.norm_w, f32, 1.f, d.norm_eps, h, l.w_in_tiled ? hb : nullptr, R, W, stream));
+    // (layers after the first find their normed input ready: the residual update of the layer
+    // before wrote it)
+    if (li == 0)
+      SQ_TRY(sd_rmsnorm_rows(x, nullptr, l.norm_w, f32, 1.f, d.norm_eps, h, l.w_in_tiled ? hb : nullptr, R, W, stream));
     // every matrix that reads h, in one product: q k v g | residual gates | ff gate, up | low-rank decay
     SQ_TRY(seq_linear(l.w_in, l.w_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, ld, R, c.total, W, wide_ws,
                       w.wide_bytes, stream));
@@ -1053,8 +1100,15 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
       SQ_TRY(seq_linear(l.w_down, l.w_down_tiled, f32, proj + c.gate, proj + c.up, ld, actb, l.ff, nullptr, ffo, W,
                         R, W, l.ff, wide_ws, w.wide_bytes, stream));
     }
-    SQ_TRY(sd_gated_residual(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, l.r1_bias,
-                             l.ff > 0 ? l.r2_bias : nullptr, mix, l.ff > 0 ? ffo : nullptr, R, W, stream));
+    if (li + 1 < d.n_layers) {
+      const sd_seq_layer& nx = m->layers[li + 1];
+      SQ_TRY(sd_gated_residual_norm(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, l.r1_bias,
+                                    l.ff > 0 ? l.r2_bias : nullptr, mix, l.ff > 0 ? ffo : nullptr, R, W, nx.norm_w,
+                                    f32, 1.f, d.norm_eps, h, nx.w_in_tiled ? hb : nullptr, stream));
+    } else {
+      SQ_TRY(sd_gated_residual(x, proj + c.r1, l.ff > 0 ? proj + c.r2 : nullptr, ld, l.r1_bias,
+                               l.ff > 0 ? l.r2_bias : nullptr, mix, l.ff > 0 ? ffo : nullptr, R, W, stream));
+    }
     if (b->layer_out) {
       const hipError_t e = hipMemcpyAsync(b->layer_out + (size_t)li * R * W, x, (size_t)R * W * sizeof(float),
                                           hipMemcpyDeviceToDevice, st);

@@ -1486,6 +1486,9 @@ extern "C" int sd_window_pool_attention(const float*, int64_t, const void*, cons
 }
 extern "C" int sd_gated_residual(float*, const float*, const float*, int64_t, const float*, const float*,
                                  const float*, const float*, int, int, sd_stream_t) { UNSUPPORTED("sd_gated_residual"); }
+extern "C" int sd_gated_residual_norm(float*, const float*, const float*, int64_t, const float*, const float*,
+                                      const float*, const float*, int, int, const void*, int, float, float, float*,
+                                      void*, sd_stream_t) { UNSUPPORTED("sd_gated_residual_norm"); }
 extern "C" int sd_relu_mul_rows(const float*, const float*, int64_t, void*, int, int, sd_stream_t) {
   UNSUPPORTED("sd_relu_mul_rows");
 }

@@ -1161,6 +1161,19 @@ def gated_residual(x, z1, a, z2=None, b=None, c1=None, c2=None) -> None:
                                              x.shape[0], x.shape[1], _stream()), "sd_gated_residual")
 
 
+def gated_residual_norm(x, z1, a, norm_w, eps, z2=None, b=None, c1=None, c2=None, offset=1.0):
+    """gated_residual, then the RMS norm of the updated rows: returns (h f32, h bf16)."""
+    for t, nm in ((x, "x"), (z1, "z1"), (a, "a")):
+        _f32(t, nm)
+    h = torch.empty_like(x)
+    h_b = torch.empty_like(x, dtype=torch.bfloat16)
+    _lib.check(_lib.load().sd_gated_residual_norm(_p(x), _p(z1), _p(z2), x.shape[1], _p(c1), _p(c2), _p(a), _p(b),
+                                                  x.shape[0], x.shape[1], _p(norm_w), _wkind(norm_w, "norm_w"),
+                                                  float(offset), float(eps), _p(h), _p(h_b), _stream()),
+               "sd_gated_residual_norm")
+    return h, h_b
+
+
 def relu_mul_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """bf16(relu(gate) * up) for f32 [rows, F] inputs."""
     _f32(gate, "gate")
