@@ -493,6 +493,32 @@ def test_long_decoding():
     assert rel(torch.cat(rows), oracle_logits(cfg, st, toks)[20:]) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_steps_replayed_as_graphs(dtype):
+    """Decoding steps of one shape replay a captured graph from their third occurrence on; between
+    the replays other work runs (a prompt joins, a request leaves, the batch changes shape and
+    comes back).  Every step's logits equal those of an engine that launches kernel by kernel."""
+    cfg = SHAPES["three_kinds"]
+    _, a = build(cfg, dtype, use_graph=True)
+    _, b = build(cfg, dtype, use_graph=False)
+    toks = [prompt(cfg, 40, i) for i in range(3)]
+
+    def both(entries):
+        x, y = a.step(entries).cpu(), b.step(entries).cpu()
+        assert torch.equal(x, y)
+
+    both([("r0", toks[0][:9], [8]), ("r1", toks[1][:3], [])])
+    for t in range(9, 20):
+        both([("r0", [toks[0][t]], [0]), ("r1", [toks[1][t - 6]], [0])])
+    both([("r2", toks[2][:17], [16]), ("r0", [toks[0][20]], [0])])          # a prompt beside a decoded token
+    for t in range(21, 30):
+        both([("r0", [toks[0][t]], [0]), ("r1", [toks[1][t - 7]], []), ("r2", [toks[2][t - 4]], [0])])
+    a.finish("r1"), b.finish("r1")
+    for t in range(30, 40):
+        both([("r2", [toks[2][t - 4]], [0]), ("r0", [toks[0][t]], [0])])    # the two-request shape again
+    assert a.graph_replays >= 20 and b.graph_replays == 0
+
+
 def test_greedy_generation_through_worker_and_scheduler():
     from vllm_omni_draft_amd import config, weights
     from vllm_omni_draft_amd.scheduler import SpecDecodeScheduler

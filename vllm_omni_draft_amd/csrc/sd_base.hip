@@ -1,5 +1,5 @@
-// What every part of the library needs: the per-thread error text, the version and the device
-// query.  (Its own object, so that a build of a subset of the library links without the rest.)
+// What every part of the library needs: the per-thread error text, the version, the device
+// query, and the hipGraph capture helpers with which a step of fixed shape replays as one launch.  (Its own object, so that a build of a subset of the library links without the rest.)
 #include <stdarg.h>
 #include <string.h>
 
@@ -44,5 +44,57 @@ extern "C" int sd_device_info(int* cu_count, char* name, size_t n) {
     name[n - 1] = '\0';
   }
   return SD_OK;
+}
+
+
+// ------------------------------------------------------------------ stream capture
+struct sd_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+
+extern "C" int sd_graph_begin(sd_stream_t stream) {
+  hipError_t e = hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    sd_set_error("sd_graph_begin: %s", hipGetErrorString(e));
+    return SD_ERR_HIP;
+  }
+  return SD_OK;
+}
+
+extern "C" int sd_graph_end(sd_stream_t stream, sd_graph** out) {
+  SD_REQUIRE(out, SD_ERR_INVALID, "sd_graph_end: null out");
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture((hipStream_t)stream, &g);
+  if (e != hipSuccess || !g) {
+    sd_set_error("sd_graph_end: capture failed: %s", hipGetErrorString(e));
+    return SD_ERR_HIP;
+  }
+  hipGraphExec_t ex = nullptr;
+  e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    sd_set_error("sd_graph_end: instantiate failed: %s", hipGetErrorString(e));
+    return SD_ERR_HIP;
+  }
+  *out = new sd_graph{g, ex};
+  return SD_OK;
+}
+
+extern "C" int sd_graph_launch(sd_graph* g, sd_stream_t stream) {
+  SD_REQUIRE(g, SD_ERR_INVALID, "sd_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch(g->exec, (hipStream_t)stream);
+  if (e != hipSuccess) {
+    sd_set_error("sd_graph_launch: %s", hipGetErrorString(e));
+    return SD_ERR_HIP;
+  }
+  return SD_OK;
+}
+
+extern "C" void sd_graph_destroy(sd_graph* g) {
+  if (!g) return;
+  (void)hipGraphExecDestroy(g->exec);   // nothing to report to: the handle is gone either way
+  (void)hipGraphDestroy(g->graph);
+  delete g;
 }
 

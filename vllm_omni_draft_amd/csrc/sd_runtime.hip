@@ -1,7 +1,6 @@
 // Host runtime of the library: the decoder-model
 // forward pass (a fixed sequence of kernel launches on the caller's stream,
-// no synchronisation, no allocation) and hipGraph capture helpers so that a
-// whole speculative step replays as one launch.
+// no synchronisation, no allocation) and the tensor-parallel group.
 #include <stdarg.h>
 #include <string.h>
 
@@ -448,56 +447,6 @@ extern "C" int sd_model_forward(sd_model* m, const sd_kv_cache* kv, const sd_for
     SD_TRY(sd_argmax_partial(a->logits, lm_vocab, a->argmax_val, a->argmax_idx, rows, lm_vocab, stream));
   }
   return SD_OK;
-}
-
-struct sd_graph {
-  hipGraph_t graph;
-  hipGraphExec_t exec;
-};
-
-extern "C" int sd_graph_begin(sd_stream_t stream) {
-  hipError_t e = hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed);
-  if (e != hipSuccess) {
-    sd_set_error("sd_graph_begin: %s", hipGetErrorString(e));
-    return SD_ERR_HIP;
-  }
-  return SD_OK;
-}
-
-extern "C" int sd_graph_end(sd_stream_t stream, sd_graph** out) {
-  SD_REQUIRE(out, SD_ERR_INVALID, "sd_graph_end: null out");
-  hipGraph_t g = nullptr;
-  hipError_t e = hipStreamEndCapture((hipStream_t)stream, &g);
-  if (e != hipSuccess || !g) {
-    sd_set_error("sd_graph_end: capture failed: %s", hipGetErrorString(e));
-    return SD_ERR_HIP;
-  }
-  hipGraphExec_t ex = nullptr;
-  e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
-  if (e != hipSuccess) {
-    (void)hipGraphDestroy(g);
-    sd_set_error("sd_graph_end: instantiate failed: %s", hipGetErrorString(e));
-    return SD_ERR_HIP;
-  }
-  *out = new sd_graph{g, ex};
-  return SD_OK;
-}
-
-extern "C" int sd_graph_launch(sd_graph* g, sd_stream_t stream) {
-  SD_REQUIRE(g, SD_ERR_INVALID, "sd_graph_launch: null graph");
-  hipError_t e = hipGraphLaunch(g->exec, (hipStream_t)stream);
-  if (e != hipSuccess) {
-    sd_set_error("sd_graph_launch: %s", hipGetErrorString(e));
-    return SD_ERR_HIP;
-  }
-  return SD_OK;
-}
-
-extern "C" void sd_graph_destroy(sd_graph* g) {
-  if (!g) return;
-  (void)hipGraphExecDestroy(g->exec);   // nothing to report to: the handle is gone either way
-  (void)hipGraphDestroy(g->graph);
-  delete g;
 }
 
 // ------------------------------------------------------------------ tensor-parallel group

@@ -10,6 +10,7 @@ models are served without speculation: one token per sequence and step.
 """
 from __future__ import annotations
 
+import ctypes as C
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -27,6 +28,12 @@ class SeqEngineConfig:
     max_tokens: int = 4096       # tokens the page pool holds (window layers), over all live requests
     max_seq_len: int = 0         # longest sequence; 0: max_tokens
     max_rows: int = 2048         # token rows per native pass; a larger step runs as several passes
+    # Steps that bring one token for each of their requests (decoding) replay as one hipGraph per
+    # (requests, wanted rows): the pass reads tokens, positions, slots and page tables from device
+    # buffers at fixed addresses, so only their contents change between replays.  The first step
+    # of a shape runs launch by launch, the second is captured.
+    use_graph: bool = True
+    graph_max_rows: int = 64
 
     @property
     def max_batch(self) -> int:  # the name the scheduler reads
@@ -56,6 +63,9 @@ class SeqEngine:
         self.model = SeqModel(weights, self.cache)
         self.seqs: Dict[str, _Seq] = {}
         self.passes = 0
+        self.stream = torch.cuda.Stream(device=self.device)   # (a capture needs a stream of its own)
+        self._graphs: Dict[Tuple[int, int], dict] = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ requests
     def has(self, request_id: str) -> bool:
@@ -117,6 +127,15 @@ class SeqEngine:
         for i, (_, _, w) in enumerate(plan):
             out_at[i] = acc
             acc += len(w)
+        torch.cuda.current_stream(self.device).synchronize()   # the caller's work on its own stream
+        with torch.cuda.stream(self.stream):
+            self._run_passes(plan, done, out_at, logits, trace)
+        self.stream.synchronize()
+        for s, t, _ in plan:
+            s.n += len(t)
+        return (logits, trace) if layer_out else logits
+
+    def _run_passes(self, plan, done, out_at, logits, trace) -> None:
         while any(done[i] < len(plan[i][1]) for i in range(len(plan))):
             room = self.cfg.max_rows
             toks: List[int] = []
@@ -142,13 +161,62 @@ class SeqEngine:
                 room -= hi - lo
                 done[i] = hi
             self._run_pass(toks, pos, slot, ents, out_rows, out_dst, logits, trace)
-        for s, t, _ in plan:
-            s.n += len(t)
-        return (logits, trace) if layer_out else logits
+
+    def _drop_graphs(self) -> None:
+        lib = _lib.load()
+        for g in self._graphs.values():
+            if g["graph"] is not None:
+                lib.sd_graph_destroy(g["graph"])
+        self._graphs = {}
+
+    def __del__(self):
+        try:
+            self._drop_graphs()
+        except Exception:
+            pass
+
+    def _run_graph_pass(self, host, R, E, O, out_dst, logits) -> bool:
+        """A decode-shaped pass through its graph; False if this shape's graph is not there yet."""
+        V = self.model_cfg.vocab
+        lib = _lib.load()
+        g = self._graphs.get((R, O))
+        if g is None:                       # first time: buffers; the pass itself runs launch by launch
+            self._graphs[(R, O)] = {"batch": torch.empty(host.numel(), dtype=torch.int32, device=self.device),
+                                    "logits": torch.empty(max(O, 1), V, dtype=torch.float32, device=self.device),
+                                    "graph": None, "workspace": None}
+            return False
+        dev = g["batch"]
+        if g["graph"] is None or g["workspace"] != self.model.workspace.data_ptr():
+            if g["graph"] is not None:      # the workspace grew since: its address is in the graph
+                lib.sd_graph_destroy(g["graph"])
+                g["graph"] = None
+            self.model._ensure_workspace(R, O)
+            handle = C.c_void_p()
+            stream = ops._stream()
+            _lib.check(lib.sd_graph_begin(stream), "sd_graph_begin")
+            try:
+                self.model.forward(R, E, dev[0:R], dev[R:2 * R], dev[2 * R:3 * R], dev[3 * R:3 * R + 4 * E], O,
+                                   dev[3 * R + 4 * E:] if O else None, g["logits"] if O else None, None)
+            finally:
+                rc = lib.sd_graph_end(stream, C.byref(handle))
+            _lib.check(rc, "sd_graph_end")
+            g["graph"], g["workspace"] = handle, self.model.workspace.data_ptr()
+        dev.copy_(host)
+        _lib.check(lib.sd_graph_launch(g["graph"], ops._stream()), "sd_graph_launch")
+        if O and out_dst == list(range(out_dst[0], out_dst[0] + O)):
+            logits[out_dst[0]:out_dst[0] + O].copy_(g["logits"][:O])
+        elif O:
+            logits[torch.tensor(out_dst, device=self.device)] = g["logits"][:O]
+        self.graph_replays += 1
+        self.passes += 1
+        return True
 
     def _run_pass(self, toks, pos, slot, ents, out_rows, out_dst, logits, trace) -> None:
         R, E, O = len(toks), len(ents) // 4, len(out_rows)
         host = torch.tensor(toks + pos + slot + ents + out_rows, dtype=torch.int32)
+        if self.cfg.use_graph and trace is None and R == E and R <= self.cfg.graph_max_rows:
+            if self._run_graph_pass(host, R, E, O, out_dst, logits):
+                return
         dev = host.to(self.device)
         a = dev[0:R]
         b = dev[R:2 * R]
