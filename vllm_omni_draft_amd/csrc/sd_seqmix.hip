@@ -3,7 +3,7 @@
 // key channel computed from the input), sliding-window attention with pooled blocks and sigmoid
 // weights, offset RMS norms, partial rotary embeddings in both pair layouts, gated residuals.
 //
-// Arithmetic contract.  Activations travel as f32 buffers; with bf16 weights the operands of the
+// Arithmetic.  Activations travel as f32 buffers; with bf16 weights the operands of the
 // matrix products (norm outputs, gated mixer outputs, feed-forward activations) are rounded to
 // bf16 values when they are stored, and keys / values are stored in the cache as bf16.  Norms,
 // angles, scores and weights, decays, the recurrent state and the residual sum are f32 always.
@@ -199,11 +199,15 @@ __global__ void head_prep_kernel(float* __restrict__ q, float* __restrict__ k, c
   }
 }
 
+// Element-wise kernels take (row, block of kColsPerBlock columns) per workgroup: a few rows of a
+// decode step still spread over many compute units.
+constexpr int kColsPerBlock = 1024;
 // decay[r, c] = sigmoid(z[r, c])^(1/tau) = exp(-softplus(-z) / tau)
 __global__ void sigmoid_power_kernel(const float* __restrict__ z, int64_t ldz, float inv_tau,
                                      float* __restrict__ out, int n_cols) {
   const int r = blockIdx.x;
-  for (int c = threadIdx.x; c < n_cols; c += blockDim.x) {
+  const int c_end = (blockIdx.y + 1) * kColsPerBlock < n_cols ? (blockIdx.y + 1) * kColsPerBlock : n_cols;
+  for (int c = blockIdx.y * kColsPerBlock + threadIdx.x; c < c_end; c += blockDim.x) {
     const float x = z[(size_t)r * ldz + c];
     const float log_sig = x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
     out[(size_t)r * n_cols + c] = expf(log_sig * inv_tau);
@@ -602,7 +606,8 @@ __global__ void gated_residual_kernel(float* __restrict__ x, const float* __rest
                                       const float* __restrict__ c2, const float* __restrict__ a,
                                       const float* __restrict__ b, int W) {
   const int r = blockIdx.x;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+  const int c_end = (blockIdx.y + 1) * kColsPerBlock < W ? (blockIdx.y + 1) * kColsPerBlock : W;
+  for (int c = blockIdx.y * kColsPerBlock + threadIdx.x; c < c_end; c += blockDim.x) {
     float add = sigmoid_f(z1[(size_t)r * ldz + c] + (c1 ? c1[c] : 0.f)) * a[(size_t)r * W + c];
     if (b) add += sigmoid_f(z2[(size_t)r * ldz + c] + (c2 ? c2[c] : 0.f)) * b[(size_t)r * W + c];
     x[(size_t)r * W + c] += add;
@@ -641,7 +646,8 @@ __global__ void gated_residual_norm_kernel(float* __restrict__ x, const float* _
 __global__ void relu_mul_rows_kernel(const float* __restrict__ gate, const float* __restrict__ up, int64_t ld,
                                      bf16_t* __restrict__ out, int F) {
   const int r = blockIdx.x;
-  for (int c = threadIdx.x; c < F; c += blockDim.x)
+  const int c_end = (blockIdx.y + 1) * kColsPerBlock < F ? (blockIdx.y + 1) * kColsPerBlock : F;
+  for (int c = blockIdx.y * kColsPerBlock + threadIdx.x; c < c_end; c += blockDim.x)
     out[(size_t)r * F + c] = (bf16_t)(fmaxf(gate[(size_t)r * ld + c], 0.f) * up[(size_t)r * ld + c]);
 }
 
@@ -712,7 +718,8 @@ extern "C" int sd_head_prep(float* q, float* k, const float* v, int64_t ld, cons
 extern "C" int sd_sigmoid_power(const float* z, int64_t ldz, float tau, float* out, int n_rows, int n_cols,
                                 sd_stream_t stream) {
   SD_REQUIRE(z && out && n_rows >= 1 && n_cols >= 1 && tau > 0.f, SD_ERR_INVALID, "sd_sigmoid_power: bad argument");
-  sigmoid_power_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(z, ldz, 1.f / tau, out, n_cols);
+  sigmoid_power_kernel<<<dim3(n_rows, (n_cols + kColsPerBlock - 1) / kColsPerBlock), 256, 0, (hipStream_t)stream>>>(
+      z, ldz, 1.f / tau, out, n_cols);
   SD_CHECK_LAUNCH("sd_sigmoid_power");
   return SD_OK;
 }
@@ -837,7 +844,8 @@ extern "C" int sd_gated_residual(float* x, const float* z1, const float* z2, int
                                  const float* c2, const float* a, const float* b, int n_rows, int W,
                                  sd_stream_t stream) {
   SD_REQUIRE(x && z1 && a && (!b || z2) && n_rows >= 1 && W >= 1, SD_ERR_INVALID, "sd_gated_residual: bad argument");
-  gated_residual_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(x, z1, z2, ldz, c1, c2, a, b, W);
+  gated_residual_kernel<<<dim3(n_rows, (W + kColsPerBlock - 1) / kColsPerBlock), 256, 0, (hipStream_t)stream>>>(
+      x, z1, z2, ldz, c1, c2, a, b, W);
   SD_CHECK_LAUNCH("sd_gated_residual");
   return SD_OK;
 }
@@ -863,7 +871,8 @@ extern "C" int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, 
                                 int F, sd_stream_t stream) {
   SD_REQUIRE(gate && up && out_bf16 && n_rows >= 1 && F >= 1 && ld >= F, SD_ERR_INVALID,
              "sd_relu_mul_rows: bad argument");
-  relu_mul_rows_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(gate, up, ld, (bf16_t*)out_bf16, F);
+  relu_mul_rows_kernel<<<dim3(n_rows, (F + kColsPerBlock - 1) / kColsPerBlock), 256, 0, (hipStream_t)stream>>>(
+      gate, up, ld, (bf16_t*)out_bf16, F);
   SD_CHECK_LAUNCH("sd_relu_mul_rows");
   return SD_OK;
 }
