@@ -254,7 +254,8 @@ class _AttnBed:
 
 
 @pytest.mark.parametrize("H,G,dk,dv,window,pool", [(2, 1, 16, 16, 9, 4), (6, 3, 24, 40, 7, 5), (1, 1, 8, 12, 1, 1),
-                                                   (4, 4, 16, 8, 20, 32), (2, 1, 72, 136, 33, 3), (2, 2, 8, 200, 40, 16)])
+                                                   (4, 4, 16, 8, 20, 32), (2, 1, 72, 136, 33, 3), (2, 2, 8, 200, 40, 16),
+                                                   (12, 1, 16, 24, 11, 2), (16, 1, 8, 8, 5, 3), (20, 2, 250, 256, 6, 7)])
 @pytest.mark.parametrize("step", ["prompt", "decode", "portions"])
 def test_window_pool_attention_random(H, G, dk, dv, window, pool, step):
     """Random keys and values over 150 positions: every position against the plain sum, with the

@@ -397,7 +397,7 @@ __global__ void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __res
 // Phase 2, a wave per key, lanes over value columns: the weighted sum.  Keys are taken in the
 // order pooled blocks, then tokens, whatever the batch: a row's bits depend on its position only.
 constexpr int kAttnTile = 256;
-constexpr int kAttnBatch = 8;   // value rows a wave has in flight
+constexpr int kAttnBatch = 8;   // value rows a wave has in flight (twice as many when a lane holds <= 2 columns)
 constexpr int kAttnLoads = 16;  // 16-byte pieces of a key row a thread has in flight
 constexpr int kAttnSplitRows = 64;  // batches of at most this many rows may split their keys over workgroups
 
@@ -528,18 +528,19 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(
     // tile's pooled keys come first, then its tokens: each loop reads one element type, with
     // unguarded loads on clamped addresses.
     const int nb_here = n_blocks - base < 0 ? 0 : (n_blocks - base < n_here ? n_blocks - base : n_here);
+    constexpr int kBatch = NC <= 2 ? 2 * kAttnBatch : kAttnBatch;
     auto sweep = [&](int lo, int hi, auto load_row) {
-      for (int kk0 = lo + wave; kk0 < hi; kk0 += 4 * kAttnBatch) {
-        float vf[kAttnBatch][NC];
+      for (int kk0 = lo + wave; kk0 < hi; kk0 += 4 * kBatch) {
+        float vf[kBatch][NC];
 #pragma unroll
-        for (int u = 0; u < kAttnBatch; ++u) {
+        for (int u = 0; u < kBatch; ++u) {
           const int kk = kk0 + 4 * u < hi ? kk0 + 4 * u : hi - 1;
           const size_t at = vat[kk];
 #pragma unroll
           for (int m = 0; m < NC; ++m) vf[u][m] = load_row(at, lane + 64 * m < dv ? lane + 64 * m : dv - 1);
         }
 #pragma unroll
-        for (int u = 0; u < kAttnBatch; ++u) {
+        for (int u = 0; u < kBatch; ++u) {
           const int kk = kk0 + 4 * u;
           if (kk < hi) {
 #pragma unroll
