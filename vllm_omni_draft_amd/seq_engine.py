@@ -268,7 +268,6 @@ class SeqWorker:
                                                          max_seq_len=c.max_model_len))
 
     def _sample(self, logits: torch.Tensor, rids: List[str]) -> List[int]:
-        from .spec_decode_worker import SamplingParams  # noqa: F401  (the carrier the requests hold)
         reqs = [self._req[r] for r in rids]
         temps = [r["sp"].temperature or 0.0 for r in reqs]
         if not any(t > 0 for t in temps):
