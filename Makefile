@@ -2,7 +2,7 @@
 HIPCC ?= /opt/rocm/bin/hipcc
 ARCH  ?= gfx950
 CSRC  := vllm_omni_draft_amd/csrc
-SRCS  := $(CSRC)/sd_base.hip $(CSRC)/sd_runtime.hip $(CSRC)/sd_sampling.hip $(CSRC)/sd_linear.hip $(CSRC)/sd_linear_wide.hip $(CSRC)/sd_attention.hip $(CSRC)/sd_ipc.hip $(CSRC)/sd_chain.hip $(CSRC)/sd_draft_layer.hip $(CSRC)/sd_seqmix.hip
+SRCS  := $(CSRC)/sd_base.hip $(CSRC)/sd_runtime.hip $(CSRC)/sd_sampling.hip $(CSRC)/sd_linear.hip $(CSRC)/sd_linear_wide.hip $(CSRC)/sd_attention.hip $(CSRC)/sd_ipc.hip $(CSRC)/sd_chain.hip $(CSRC)/sd_draft_layer.hip $(CSRC)/sd_seqmix.hip $(CSRC)/sd_seqmix_hybrid.hip
 OBJS  := $(SRCS:.hip=.o)
 LIB   := vllm_omni_draft_amd/libsd_amd.so
 EXTRA ?=
@@ -35,7 +35,7 @@ $(LIB): $(OBJS)
 # run in a fresh checkout that should not wait for every kernel family to compile.  The package
 # loads it only where the whole library has not been built.
 SEQ_LIB  := vllm_omni_draft_amd/libsd_seq.so
-SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_sampling.o $(CSRC)/sd_linear.o $(CSRC)/sd_linear_wide.o
+SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_seqmix_hybrid.o $(CSRC)/sd_sampling.o $(CSRC)/sd_linear.o $(CSRC)/sd_linear_wide.o
 $(SEQ_LIB): $(SEQ_OBJS)
 	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(SEQ_OBJS)
 seq: $(SEQ_LIB)

@@ -1110,11 +1110,116 @@ int sd_gated_residual_norm(float* x, const float* z1, const float* z2, int64_t l
 int sd_relu_mul_rows(const float* gate, const float* up, int64_t ld, void* out_bf16, int n_rows,
                      int F, sd_stream_t stream);
 
+/* ---- mechanisms of hybrid decoders: softmax attention over a window with kept first tokens,
+ * latent (low-rank) keys and values, a state-space recurrence with a scalar decay per head,
+ * routed experts, norms on a sublayer's output.  Same conventions as above.               */
+
+/* x[r] = table[tokens[r]] * scale (+ bigram[row] when bigram != NULL: row = (prev * mul_prev +
+ * tok * mul_cur) mod buckets, or row `buckets` when prev_tokens[r] < 0: a sequence's first
+ * token).  x_bf16 (or NULL): the same rows as bf16.  The row index is formed in 64 bits.    */
+int sd_embed_hashed(const int32_t* tokens, const int32_t* prev_tokens, const void* table,
+                    const void* bigram, int w_f32, float scale, int buckets, int mul_prev,
+                    int mul_cur, float* x, void* x_bf16, int n_rows, int W, int vocab,
+                    sd_stream_t stream);
+/* Columns [0, width) of every row (row stride ldx) in `parts` equal parts, each divided by its
+ * own root mean square (eps inside the root) and multiplied by w[c] (w [width], or NULL).
+ * gate != NULL: the input is x * silu(gate) (row stride ldg), taken before the norm.  out row
+ * stride ldo (out may be x); out_bf16 (or NULL) row stride ldob.                             */
+int sd_rmsnorm_parts(const float* x, int64_t ldx, const float* gate, int64_t ldg, const void* w,
+                     int w_f32, float eps, float* out, int64_t ldo, void* out_bf16, int64_t ldob,
+                     int n_rows, int width, int parts, int round_bf16_out, sd_stream_t stream);
+/* In place, per (row, head): channels offset + 2i and offset + 2i + 1 (rot_layout 1) or offset + i
+ * and offset + i + rot_dims/2 (0), i < rot_dims/2, of the vector at x + row*ld + head*head_stride
+ * are turned by row_pos * inv_freq[i]; cos and sin are multiplied by `mag`.                  */
+int sd_rope_rows(float* x, int64_t ld, const int32_t* row_pos, int n_rows, int heads,
+                 int head_stride, int offset, int rot_dims, int rot_layout, const double* inv_freq,
+                 float mag, sd_stream_t stream);
+/* The same turn on the way from src to dst: per (row, head) the n channels at src + row*ld_src +
+ * head*src_head_stride + src_offset go to dst + row*ld_dst + head*dst_head_stride + dst_offset,
+ * the first rot_dims of them turned.  src and dst are the same place or do not overlap.       */
+int sd_rope_copy_rows(const float* src, int64_t ld_src, int src_head_stride, int src_offset,
+                      float* dst, int64_t ld_dst, int dst_head_stride, int dst_offset,
+                      const int32_t* row_pos, int n_rows, int heads, int n, int rot_dims,
+                      int rot_layout, const double* inv_freq, float mag, sd_stream_t stream);
+/* Appends key rows k [rows, G*dk] (row stride ldk) and, unless v == NULL, value rows
+ * v [rows, G*dv] to pages of `page` tokens: row (page, head, token) of dk / dv elements.    */
+int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, void* k_cache,
+                    void* v_cache, int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
+                    const int32_t* block_tables, int max_blocks, int page, int n_rows, int G,
+                    int dk, int dv, sd_stream_t stream);
+/* Softmax attention over the cache sd_cache_append fills.  The row at position i sees j <= i
+ * with i - j < window or j < keep_first; out[r, h] = sum_j softmax_j(q.k_j * scale) v_j, query
+ * head h reads kv head h / (H/G).  v_cache == NULL: a value row is the first dv channels of its
+ * key row (latent attention: keys and values share one cached row).  Keys are taken in the
+ * order kept tokens, then window, in tiles of 256 with a running maximum; dv <= 512.
+ * out_bf16 (or NULL): the same as bf16.                                                     */
+int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache,
+                                const void* v_cache, int cache_f32, const int32_t* row_pos,
+                                const int32_t* row_slot, const int32_t* block_tables,
+                                int max_blocks, int page, int n_rows, int H, int G, int dk, int dv,
+                                int window, int keep_first, float scale, float* out,
+                                void* out_bf16, sd_stream_t stream);
+/* y[z][M, N] = x[z][M, K] w[z][N, K]^T for z < batch: x + z*bx (row stride ldx), w + z*bw,
+ * y + z*by (row stride ldy); y_bf16 (or NULL) laid out as y.                                */
+int sd_matmul_rows_batched(const float* x, int64_t ldx, int64_t bx, const void* w, int w_f32,
+                           int64_t bw, float* y, int64_t ldy, int64_t by, void* y_bf16, int M,
+                           int N, int K, int batch, sd_stream_t stream);
+/* Causal convolution per channel over each entry's tokens, then silu (act != 0):
+ * out[r, c] = act(b[c] + sum_j w[c, taps-1-j] * in(r, j)), in(r, j) the input j tokens before
+ * row r: from x (row stride ldx), from the slot's state (the taps-1 inputs before the entry,
+ * conv_state [slots, taps-1, C] f32, oldest first), or zero before the sequence's start.  Then
+ * the state is moved on to the entry's last taps-1 inputs.  w [C, taps], b [C] or NULL.      */
+int sd_causal_conv_rows(const float* x, int64_t ldx, const void* w, const void* b, int w_f32,
+                        float* conv_state, const int32_t* row_pos, const int32_t* row_slot,
+                        const int32_t* entries, int n_entries, float* out, int64_t ldo, int n_rows,
+                        int C, int taps, int act, sd_stream_t stream);
+/* step[r, h] = softplus(dt[r, h] + dt_bias[h]);  decay[r, h] = exp(-exp(a_log[h]) * step).   */
+int sd_ssd_steps(const float* dt, int64_t ld, const void* dt_bias, const void* a_log, int w_f32,
+                 float* step, float* decay, int n_rows, int H, sd_stream_t stream);
+/* The recurrence of sd_decay_scan with a scalar decay per (row, head):
+ *   S <- decay[r, h] S + (k_scale[r, h] k_t) v_t^T,   o_t = S^T q_t + skip[h] v_t,
+ * q, k [rows, Gq*dk] (row stride ldqk; head h reads group h / (H/Gq)), v [rows, H*dv] (row
+ * stride ldv), k_scale [rows, H] or NULL, skip [H] (model element type) or NULL.            */
+int sd_decay_scan_rows(const float* q, const float* k, int64_t ldqk, const float* v, int64_t ldv,
+                       const float* decay, const float* k_scale, const void* skip, int w_f32,
+                       float* state, const int32_t* entries, int n_entries, float* out, int H,
+                       int Gq, int dk, int dv, sd_stream_t stream);
+/* Routed experts.  logits [rows, E] (row stride ld): score = sigmoid (score_kind 0) or softmax
+ * over the experts (1); the `top` largest (lowest index first among equals) go to sel_expert /
+ * sel_weight [rows, top], weights divided by their sum when renorm.                          */
+int sd_moe_route(const float* logits, int64_t ld, int32_t* sel_expert, float* sel_weight,
+                 int n_rows, int E, int top, int score_kind, int renorm, sd_stream_t stream);
+/* Bytes of scratch sd_moe_experts needs.                                                   */
+size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W);
+/* out[r*top + j] = down_e(act(gate_e u) * (up_e u)) for e = sel_expert[r, j], u = sel_weight *
+ * x[r] (scale_input) or u = x[r] with the result multiplied by the weight (scale_input == 0);
+ * act_kind 0: silu.  w_gate_up [E, 2F, W] (gate rows, then up rows), w_down [E, W, F]; x
+ * [rows, W]; out [rows*top, W]: the caller adds a row's `top` results.  Rows are grouped by
+ * expert on the device; nothing is read back.                                               */
+int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_expert, const float* sel_weight,
+                   const void* w_gate_up, const void* w_down, int w_f32, float* out, int n_rows,
+                   int top, int E, int F, int W, int scale_input, int act_kind, void* scratch,
+                   size_t scratch_bytes, sd_stream_t stream);
+/* x[r] += rms_norm(sa * (a[r*n_a] + ... + a[r*n_a + n_a - 1]) + sb * b[r]) * w  (b may be NULL;
+ * a [rows*n_a, W], b [rows, W], w [W] plain).  x_bf16 (or NULL): the updated rows as bf16.   */
+int sd_postnorm_residual(float* x, const float* a, int n_a, float sa, const float* b, float sb,
+                         const void* w, int w_f32, float eps, void* x_bf16, int n_rows, int W,
+                         sd_stream_t stream);
+/* x[r, c] *= s                                                                             */
+int sd_scale_rows(float* x, int64_t ld, float s, int n_rows, int n_cols, sd_stream_t stream);
+
 typedef enum {
   SD_MIX_HEAD_DECAY = 0,    /* recurrence with a fixed decay per head (retention) */
   SD_MIX_CHANNEL_DECAY = 1, /* recurrence with an input-dependent decay per key channel */
-  SD_MIX_WINDOW_POOL = 2    /* sd_window_pool_attention */
+  SD_MIX_WINDOW_POOL = 2,   /* sd_window_pool_attention */
+  SD_MIX_LATENT = 3,        /* softmax window attention over latent keys / values */
+  SD_MIX_SOFTMAX_SSD = 4    /* softmax window attention and a state-space recurrence side by side */
 } sd_mixer_kind;
+
+typedef enum {
+  SD_BLOCK_GATED = 0,       /* h = norm(x); x += sigmoid(r1) mixer(h) + sigmoid(r2) ff(h) */
+  SD_BLOCK_POSTNORM = 1     /* x += norm1(mixer(x)); x += norm2(ff(x)) */
+} sd_block_kind;
 
 /* One layer: h = norm(x); x += sigmoid(r1) * mixer(h) + sigmoid(r2) * ff(h).  w_in stacks every
  * matrix that reads h, rows in this order: q [heads*dim], k [kv_heads*dim], v [kv_heads*vdim],
@@ -1153,6 +1258,41 @@ typedef struct {
   void* v_cache;
   float* pk_cache;
   float* pv_cache;
+  /* ---- SD_BLOCK_POSTNORM layers (all zero otherwise).  w_in stacks the matrices that read x:
+   * SD_MIX_LATENT: dq [q_rank], dkv [kv_rank + rot_dim]; SD_MIX_SOFTMAX_SSD: q [heads*dim],
+   * k [kv_heads*dim], v [kv_heads*vdim], ssd in [2*inner + 2*groups*state + s_heads].  norm_w is
+   * norm1 (plain weight), w_o the attention's output matrix.                                */
+  int block;
+  int keep_first;
+  const void* norm2_w;      /* [width] or NULL (no feed-forward) */
+  /* latent attention: per head `dim` unrotated and `rot_dim` rotated channels */
+  int q_rank, kv_rank, rot_dim;
+  float rot_mag;            /* factor of cos and sin */
+  const void* dq_norm_w;    /* [q_rank] */
+  const void* dkv_norm_w;   /* [kv_rank] */
+  const void* w_uq;         /* [heads*(dim+rot_dim), q_rank] */
+  const void* w_uq_tiled;
+  const void* w_uk_t;       /* [heads, kv_rank, dim]: each head's key expansion, transposed */
+  const void* w_uv;         /* [heads*vdim, kv_rank] */
+  /* softmax attention beside a state-space recurrence */
+  const void* q_norm_w;     /* [heads*dim] */
+  const void* k_norm_w;     /* [kv_heads*dim] */
+  float left_scale, right_scale;
+  int s_heads, s_vdim, s_state, s_groups, s_taps, s_norm_groups;
+  const void* conv_w;       /* [inner + 2*groups*state, taps] */
+  const void* conv_b;
+  const void* dt_bias;      /* [s_heads] */
+  const void* a_log;
+  const void* skip_d;
+  const void* s_norm_w;     /* [inner] */
+  const void* w_o2;         /* [width, inner] */
+  const void* w_o2_tiled;
+  float* conv_state;        /* [slots, taps-1, inner + 2*groups*state] */
+  /* routed experts */
+  int n_experts, top, expert_ff;
+  const void* w_router;     /* [n_experts, width] */
+  const void* w_gate_up;    /* [n_experts, 2*expert_ff, width] */
+  const void* w_down_e;     /* [n_experts, width, expert_ff] */
 } sd_seq_layer;
 
 typedef struct {
@@ -1163,6 +1303,13 @@ typedef struct {
   const void* head_tiled;  /* NULL, or the same table as SD_TILE_PLAIN tiles for the head */
   const void* final_norm_w;
   const sd_seq_layer* layers; /* copied */
+  /* SD_BLOCK_POSTNORM models: plain norm weights; otherwise zero / NULL */
+  int plain_norm;          /* the final norm's weight is plain (not stored around zero) */
+  float embed_scale;       /* 0: 1 */
+  const void* bigram;      /* [buckets + 1, width] or NULL */
+  int buckets, mul_prev, mul_cur;
+  const void* head;        /* [vocab, width] row-major, or NULL: the embedding table is the head */
+  float logit_scale;       /* 0: 1 */
 } sd_seq_model_desc;
 
 typedef struct {
@@ -1177,6 +1324,8 @@ typedef struct {
   const int32_t* out_rows; /* [n_out] rows whose logits are wanted */
   float* logits;           /* [n_out, vocab] */
   float* layer_out;        /* NULL, or [n_layers, n_rows, width]: the residual after each layer */
+  const int32_t* prev_tokens; /* [n_rows] the token before each row in its sequence, -1: none
+                                 (models with a bigram table; NULL otherwise) */
 } sd_seq_batch;
 
 typedef struct sd_seq_model sd_seq_model;

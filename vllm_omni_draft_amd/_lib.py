@@ -84,19 +84,30 @@ class SeqLayer(C.Structure):
                 ("norm_w", vp), ("w_in", vp), ("w_in_tiled", vp), ("r1_bias", vp), ("r2_bias", vp), ("w_o", vp),
                 ("w_o_tiled", vp), ("w_down", vp), ("w_down_tiled", vp), ("w_a2", vp),
                 ("b_a2", vp), ("head_decay", vp), ("head_bias", vp), ("head_norm_w", vp), ("state", vp),
-                ("k_cache", vp), ("v_cache", vp), ("pk_cache", vp), ("pv_cache", vp)]
+                ("k_cache", vp), ("v_cache", vp), ("pk_cache", vp), ("pv_cache", vp),
+                ("block", i32), ("keep_first", i32), ("norm2_w", vp),
+                ("q_rank", i32), ("kv_rank", i32), ("rot_dim", i32), ("rot_mag", C.c_float),
+                ("dq_norm_w", vp), ("dkv_norm_w", vp), ("w_uq", vp), ("w_uq_tiled", vp), ("w_uk_t", vp), ("w_uv", vp),
+                ("q_norm_w", vp), ("k_norm_w", vp), ("left_scale", C.c_float), ("right_scale", C.c_float),
+                ("s_heads", i32), ("s_vdim", i32), ("s_state", i32), ("s_groups", i32), ("s_taps", i32),
+                ("s_norm_groups", i32), ("conv_w", vp), ("conv_b", vp), ("dt_bias", vp), ("a_log", vp),
+                ("skip_d", vp), ("s_norm_w", vp), ("w_o2", vp), ("w_o2_tiled", vp), ("conv_state", vp),
+                ("n_experts", i32), ("top", i32), ("expert_ff", i32), ("w_router", vp), ("w_gate_up", vp),
+                ("w_down_e", vp)]
 
 
 class SeqModelDesc(C.Structure):
     _fields_ = [("n_layers", i32), ("width", i32), ("vocab", i32), ("weights_f32", i32),
                 ("norm_eps", C.c_float), ("embed", vp), ("head_tiled", vp), ("final_norm_w", vp),
-                ("layers", C.POINTER(SeqLayer))]
+                ("layers", C.POINTER(SeqLayer)),
+                ("plain_norm", i32), ("embed_scale", C.c_float), ("bigram", vp), ("buckets", i32),
+                ("mul_prev", i32), ("mul_cur", i32), ("head", vp), ("logit_scale", C.c_float)]
 
 
 class SeqBatch(C.Structure):
     _fields_ = [("n_rows", i32), ("n_entries", i32), ("tokens", vp), ("row_pos", vp), ("row_slot", vp),
                 ("entries", vp), ("block_tables", vp), ("max_blocks", i32), ("page", i32), ("n_out", i32),
-                ("out_rows", vp), ("logits", vp), ("layer_out", vp)]
+                ("out_rows", vp), ("logits", vp), ("layer_out", vp), ("prev_tokens", vp)]
 
 
 # name -> (restype, argtypes); every symbol include/sd_amd.h declares.
@@ -225,6 +236,22 @@ SIGNATURES = {
     "sd_gated_residual_norm": (i32, [vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, vp, i32, C.c_float, C.c_float,
                                      vp, vp, vp]),
     "sd_relu_mul_rows": (i32, [vp, vp, i64, vp, i32, i32, vp]),
+    "sd_embed_hashed": (i32, [vp, vp, vp, vp, i32, C.c_float, i32, i32, i32, vp, vp, i32, i32, i32, vp]),
+    "sd_rmsnorm_parts": (i32, [vp, i64, vp, i64, vp, i32, C.c_float, vp, i64, vp, i64, i32, i32, i32, i32, vp]),
+    "sd_rope_rows": (i32, [vp, i64, vp, i32, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
+    "sd_rope_copy_rows": (i32, [vp, i64, i32, i32, vp, i64, i32, i32, vp, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
+    "sd_cache_append": (i32, [vp, i64, vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
+    "sd_window_softmax_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32,
+                                          i32, C.c_float, vp, vp, vp]),
+    "sd_matmul_rows_batched": (i32, [vp, i64, i64, vp, i32, i64, vp, i64, i64, vp, i32, i32, i32, i32, vp]),
+    "sd_causal_conv_rows": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, i32, vp, i64, i32, i32, i32, i32, vp]),
+    "sd_ssd_steps": (i32, [vp, i64, vp, vp, i32, vp, vp, i32, i32, vp]),
+    "sd_decay_scan_rows": (i32, [vp, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, i32, vp, i32, i32, i32, i32, vp]),
+    "sd_moe_route": (i32, [vp, i64, vp, vp, i32, i32, i32, i32, i32, vp]),
+    "sd_moe_experts_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
+    "sd_moe_experts": (i32, [vp, i64, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_size_t, vp]),
+    "sd_postnorm_residual": (i32, [vp, vp, i32, C.c_float, vp, C.c_float, vp, i32, C.c_float, vp, i32, i32, vp]),
+    "sd_scale_rows": (i32, [vp, i64, C.c_float, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),
     "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32, i32]),

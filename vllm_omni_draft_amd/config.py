@@ -210,7 +210,56 @@ def rope_table(cfg: ModelConfig, device="cpu") -> torch.Tensor:
 
 # ---------------------------------------------------------------------------------------------
 # Decoders described layer by layer (recurrent and windowed mixers); served by seq_engine.SeqEngine.
-MIXER_KINDS = ("retention", "gla", "attention")
+MIXER_KINDS = ("retention", "gla", "attention", "latent_attention", "parallel")
+
+
+@dataclass
+class SsdSpec:
+    """A state-space recurrence with a scalar decay per head (the state-space-duality form):
+    S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x; x, B, C pass a causal convolution of
+    `taps` taps and silu; the output is gated by silu(z) and RMS-normed in `norm_groups` parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int = 1
+    taps: int = 4
+    norm_groups: int = 1
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    def validate(self) -> None:
+        if min(self.heads, self.vdim, self.state, self.groups, self.taps, self.norm_groups) < 1:
+            raise ValueError("state-space sizes must be positive")
+        if self.heads % self.groups or self.inner % self.norm_groups:
+            raise ValueError("state-space heads must divide into groups, and the inner size into norm groups")
+        if self.state > 256:
+            raise ValueError("a state size above 256 is not supported")
+
+
+@dataclass
+class ExpertsSpec:
+    """Routed experts as a layer's feed-forward: `top` of `experts` gated feed-forwards of width
+    `ff` per token.  score: "sigmoid" or "softmax" over the router's logits; renorm: the chosen
+    weights are divided by their sum; scale_input: the weight multiplies the expert's input
+    (else its output)."""
+    experts: int
+    top: int
+    ff: int
+    score: str = "sigmoid"
+    renorm: bool = False
+    scale_input: bool = True
+
+    def validate(self) -> None:
+        if self.experts < 1 or not 1 <= self.top <= self.experts or self.ff < 1:
+            raise ValueError(f"experts {self.experts}, top {self.top}, ff {self.ff}")
+        if self.score not in ("sigmoid", "softmax"):
+            raise ValueError(f"unknown router score {self.score!r}")
 
 
 @dataclass
@@ -219,7 +268,13 @@ class MixerSpec:
     head and rotate-half rotary positions; "gla": decayed linear attention whose decay per key
     channel comes from the input through a low-rank pair of matrices (sigmoid(z)^(1/tau));
     "attention": grouped-query attention over a sliding window plus mean-pooled blocks of the
-    tokens before it, with sigmoid weights, interleaved rotary positions and unit-norm q / k."""
+    tokens before it, with sigmoid weights, interleaved rotary positions and unit-norm q / k;
+    "latent_attention": softmax attention over a sliding window whose keys and values are
+    expanded from one cached latent of kv_rank channels per token, plus rot_dim rotated channels
+    shared by the heads (queries through a latent of q_rank channels; dim counts the unrotated
+    channels of a head); "parallel": grouped-query softmax attention without rotation, q and k
+    normed over the whole projection, over a window that also keeps the first keep_first tokens,
+    beside a state-space recurrence (ssd) on the same input, summed with two scales."""
     kind: str
     heads: int
     dim: int
@@ -234,6 +289,14 @@ class MixerSpec:
     scale: float = 1.0             # attention: factor of the scores
     window: int = 0                # attention: tokens seen, the current one included
     pool: int = 1                  # attention: tokens per pooled block
+    keep_first: int = 0            # parallel: the first tokens stay visible behind the window
+    q_rank: int = 0                # latent_attention
+    kv_rank: int = 0
+    rot_dim: int = 0               # latent_attention: rotated channels per head (behind the `dim` unrotated)
+    rot_scaling: Optional[dict] = None  # frequency blending {factor, original, fast, slow}
+    ssd: Optional[SsdSpec] = None  # parallel
+    left_scale: float = 1.0        # parallel: factor of the attention
+    right_scale: float = 1.0       # parallel: factor of the recurrence
 
     def validate(self) -> None:
         if self.kind not in MIXER_KINDS:
@@ -244,6 +307,20 @@ class MixerSpec:
                              f"vdim {self.vdim}")
         if self.rot_layout not in ("half", "interleaved"):
             raise ValueError(f"unknown rotary layout {self.rot_layout!r}")
+        if self.kind == "latent_attention":
+            if min(self.q_rank, self.kv_rank) < 1 or self.rot_dim < 0 or self.window < 1:
+                raise ValueError("latent attention needs q_rank, kv_rank >= 1, rot_dim >= 0, window >= 1")
+            if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.rot_dim:
+                raise ValueError(f"rot_dims {self.rot_dims} must be even and at most rot_dim {self.rot_dim}")
+            if self.kv_rank > 512 or self.kv_heads != self.heads:
+                raise ValueError("latent attention: kv_rank above 512, or kv_heads given")
+            return
+        if self.kind == "parallel":
+            if self.window < 1 or self.keep_first < 0 or self.rot_dims or self.ssd is None or self.vdim > 512:
+                raise ValueError("a parallel mixer needs window >= 1, keep_first >= 0, no rotation, vdim <= 512 "
+                                 "and a state-space part")
+            self.ssd.validate()
+            return
         if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.dim:
             raise ValueError(f"rot_dims {self.rot_dims} must be even and at most dim {self.dim}")
         if self.kind == "attention":
@@ -264,10 +341,32 @@ class MixerSpec:
             raise ValueError("gla needs tau > 0")
 
 
+def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
+    """(frequencies of the dims/2 pairs as float64, factor of cos and sin).  Plain: base^(-2i/dims)
+    and 1.  With scaling {factor, original, fast, slow}: pair i keeps its frequency f_i where it
+    turns fast and takes f_i / factor where it turns slowly, blended along a ramp over the pair
+    index between the pairs that make `fast` and `slow` turns over `original` positions; cos and
+    sin grow by 0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / dims)
+    if not scaling:
+        return f, 1.0
+    factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+    def pair_index(turns: float) -> float:
+        return dims * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(base))
+
+    lo = max(math.floor(pair_index(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(pair_index(float(scaling["slow"]))), dims - 1)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
+
+
 @dataclass
 class SeqLayerSpec:
     mixer: MixerSpec
     ff: int = 0                    # width of the gated feed-forward beside the mixer; 0: none
+    experts: Optional[ExpertsSpec] = None   # routed experts as the feed-forward
 
 
 @dataclass
@@ -281,14 +380,34 @@ class SeqModelConfig:
     layers: List["SeqLayerSpec"]
     norm_eps: float = 1e-5
     name: str = "custom"
+    # "gated": the layer above.  "postnorm": x += norm1(mixer(x)); x += norm2(ff(x)), plain norm
+    # weights, the sublayers read x itself; the feed-forward is a set of routed experts or absent.
+    block: str = "gated"
+    embed_scale: float = 1.0
+    bigram: Optional[dict] = None  # {buckets, mul_prev, mul_cur}: a hashed table of token pairs added to the embedding
+    tied_head: bool = True         # False: the output head is its own tensor
+    logit_scale: float = 1.0
 
     def validate(self) -> None:
         if self.width < 1 or self.vocab < 1 or not self.layers:
             raise ValueError("a model needs width, vocab and at least one layer")
+        if self.block not in ("gated", "postnorm"):
+            raise ValueError(f"unknown block {self.block!r}")
+        if self.bigram is not None and int(self.bigram["buckets"]) < 1:
+            raise ValueError("a bigram table needs buckets >= 1")
         for l in self.layers:
             l.mixer.validate()
             if l.ff < 0:
                 raise ValueError("ff must be >= 0")
+            post = l.mixer.kind in ("latent_attention", "parallel")
+            if post != (self.block == "postnorm"):
+                raise ValueError(f"mixer {l.mixer.kind!r} does not belong to a {self.block!r} model")
+            if l.experts is not None:
+                l.experts.validate()
+                if not post or l.ff:
+                    raise ValueError("routed experts are the feed-forward of a postnorm layer, and its only one")
+            elif post and l.ff:
+                raise ValueError("a postnorm layer's feed-forward is a set of routed experts")
 
     @property
     def n_layers(self) -> int:
@@ -296,16 +415,38 @@ class SeqModelConfig:
 
     def param_count(self) -> int:
         W, n = self.width, self.vocab * self.width + self.width
+        if not self.tied_head:
+            n += self.vocab * W
+        if self.bigram:
+            n += (int(self.bigram["buckets"]) + 1) * W
         for l in self.layers:
             m = l.mixer
+            if m.kind == "latent_attention":
+                n += W + W * (m.q_rank + m.kv_rank + m.rot_dim) + m.q_rank + m.kv_rank
+                n += m.heads * ((m.dim + m.rot_dim) * m.q_rank + (m.dim + m.vdim) * m.kv_rank + m.vdim * W)
+            elif m.kind == "parallel":
+                sd = m.ssd
+                n += W + (W + 1) * (m.heads * m.dim + m.kv_heads * m.dim) + W * m.kv_heads * m.vdim + m.heads * m.vdim * W
+                n += W * (2 * sd.inner + 2 * sd.groups * sd.state + sd.heads) + sd.conv_channels * (sd.taps + 1)
+                n += 3 * sd.heads + sd.inner + sd.inner * W
+            if l.experts is not None:
+                n += W + l.experts.experts * (W + 3 * l.experts.ff * W)
+            if m.kind in ("latent_attention", "parallel"):
+                continue
             n += W + W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim) + 2 * m.heads * m.vdim) + W * W + W
             n += (m.rank * (W + m.heads * m.dim) + m.heads * m.dim + m.vdim) if m.kind == "gla" else 0
             n += (3 * l.ff * W + W * W + W) if l.ff else 0
         return n
 
     def state_bytes_per_seq(self) -> int:
-        return sum(4 * l.mixer.heads * l.mixer.dim * l.mixer.vdim for l in self.layers
-                   if l.mixer.kind != "attention")
+        n = 0
+        for l in self.layers:
+            m = l.mixer
+            if m.kind == "parallel":
+                n += 4 * (m.ssd.heads * m.ssd.state * m.ssd.vdim + (m.ssd.taps - 1) * m.ssd.conv_channels)
+            elif m.kind in ("retention", "gla"):
+                n += 4 * m.heads * m.dim * m.vdim
+        return n
 
 
 def puguzen_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides) -> SeqModelConfig:
@@ -340,8 +481,58 @@ def puguzen_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides)
     return out
 
 
+def naburax_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides) -> SeqModelConfig:
+    """A Naburax config.json: latent-attention layers and layers with attention beside a
+    state-space recurrence, in any order, each normed on its sublayers' outputs, routed experts
+    as feed-forward, a scaled embedding plus a hashed table of token pairs, an untied head."""
+    layers = []
+    for i, l in enumerate(cfg["layers"]):
+        m, kind = l["mixer"], l["type"]
+        if kind == "latent_attention":
+            rot = m.get("rot") or {}
+            shape = (tensor_shapes or {}).get(f"l{i}.mix.dq")
+            spec = MixerSpec(kind=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                             q_rank=int(shape[0]) if shape is not None else int(m["q_rank"]),
+                             kv_rank=int(m["kv_rank"]), rot_dim=int(m.get("rot_dim", 0)),
+                             rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                             rot_layout="interleaved", rot_scaling=rot.get("scaling") or None,
+                             scale=float(m["scale"]), window=int(m["mask"]["size"]))
+        elif kind == "parallel":
+            a, b = m["left"], m["right"]
+            spec = MixerSpec(kind=kind, heads=int(a["heads"]), kv_heads=int(a.get("kv_heads", 0)), dim=int(a["dim"]),
+                             vdim=int(a["vdim"]), scale=float(a["scale"]), window=int(a["mask"]["size"]),
+                             keep_first=int(a["mask"].get("keep_first", 0)),
+                             ssd=SsdSpec(heads=int(b["heads"]), vdim=int(b["vdim"]), state=int(b["state"]),
+                                         groups=int(b.get("groups", 1)), taps=int(b["conv"]),
+                                         norm_groups=int(b.get("norm_groups", 1))),
+                             left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp = l.get("mlp")
+        experts = None
+        if mlp:
+            if mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported")
+            experts = ExpertsSpec(experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]),
+                                  ff=int(mlp["expert"]["ff"]))
+        layers.append(SeqLayerSpec(spec, 0, experts))
+    emb = cfg.get("embedding") or {}
+    bg = emb.get("bigram")
+    out = SeqModelConfig(arch="naburax", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers,
+                         norm_eps=float(cfg["norm"]["eps"]), name=cfg.get("architecture", "Naburax"),
+                         block="postnorm", embed_scale=float(emb.get("scale", 1.0)),
+                         bigram={k: int(bg[k]) for k in ("buckets", "mul_prev", "mul_cur")} if bg else None,
+                         tied_head=False, logit_scale=float(cfg.get("logit_scale", 1.0)))
+    for k, v in overrides.items():
+        if not hasattr(out, k):
+            raise ValueError(f"Unknown config parameter: {k}")
+        setattr(out, k, v)
+    out.validate()
+    return out
+
+
 # config.json "architecture" -> builder of a layer-list config
-SEQ_ARCHITECTURES = {"Puguzen": puguzen_config}
+SEQ_ARCHITECTURES = {"Puguzen": puguzen_config, "Naburax": naburax_config}
 
 
 def safetensors_shapes(path: str) -> dict:

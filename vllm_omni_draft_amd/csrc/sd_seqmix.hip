@@ -76,8 +76,13 @@ __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* 
 template <typename T, int BM, int BN, int TM, int TN>
 __global__ __launch_bounds__(256) void matmul_rows_kernel(
     const float* __restrict__ X, const float* __restrict__ X2, int64_t ldx, const T* __restrict__ Wt,
-    const float* __restrict__ bias, float* __restrict__ Y, int64_t ldy, int M, int N, int K, int round) {
+    const float* __restrict__ bias, float* __restrict__ Y, int64_t ldy, int M, int N, int K, int round,
+    int64_t bx = 0, int64_t bw = 0, int64_t by = 0, bf16_t* __restrict__ Yb = nullptr) {
   constexpr int BK = 16;
+  X += (size_t)blockIdx.z * bx;    // blockIdx.z: one product of a batch (operands bx / bw / by apart)
+  Wt += (size_t)blockIdx.z * bw;
+  Y += (size_t)blockIdx.z * by;
+  if (Yb) Yb += (size_t)blockIdx.z * by;
   static_assert((BM / TM) * (BN / TN) == 256, "256 threads");
   __shared__ float xs[BK][BM + 1];
   __shared__ float ws[BK][BN + 1];
@@ -126,7 +131,11 @@ __global__ __launch_bounds__(256) void matmul_rows_kernel(
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + tx * TN + j;
-      if (n < N) Y[(size_t)m * ldy + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+      if (n < N) {
+        const float o = acc[i][j] + (bias ? bias[n] : 0.f);
+        Y[(size_t)m * ldy + n] = o;
+        if (Yb) Yb[(size_t)m * ldy + n] = (bf16_t)o;
+      }
     }
   }
 }
@@ -654,13 +663,16 @@ __global__ void relu_mul_rows_kernel(const float* __restrict__ gate, const float
 
 template <typename T>
 int launch_matmul(const float* X, const float* X2, int64_t ldx, const void* Wt, const float* bias, float* Y,
-                  int64_t ldy, int M, int N, int K, int round, hipStream_t st) {
+                  int64_t ldy, int M, int N, int K, int round, hipStream_t st, int batch = 1, int64_t bx = 0,
+                  int64_t bw = 0, int64_t by = 0, bf16_t* Yb = nullptr) {
   if (M <= 16) {
-    dim3 grid((N + 127) / 128, (M + 15) / 16);
-    matmul_rows_kernel<T, 16, 128, 2, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round);
+    dim3 grid((N + 127) / 128, (M + 15) / 16, batch);
+    matmul_rows_kernel<T, 16, 128, 2, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round,
+                                                               bx, bw, by, Yb);
   } else {
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
-    matmul_rows_kernel<T, 64, 64, 4, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round);
+    dim3 grid((N + 63) / 64, (M + 63) / 64, batch);
+    matmul_rows_kernel<T, 64, 64, 4, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round,
+                                                              bx, bw, by, Yb);
   }
   SD_CHECK_LAUNCH("sd_matmul_rows");
   return SD_OK;
@@ -677,6 +689,16 @@ extern "C" int sd_matmul_rows(const float* x, const float* x2, int64_t ldx, cons
   hipStream_t st = (hipStream_t)stream;
   return w_f32 ? launch_matmul<float>(x, x2, ldx, w, bias, y, ldy, M, N, K, 0, st)
                : launch_matmul<bf16_t>(x, x2, ldx, w, bias, y, ldy, M, N, K, 1, st);
+}
+
+extern "C" int sd_matmul_rows_batched(const float* x, int64_t ldx, int64_t bx, const void* w, int w_f32, int64_t bw,
+                                      float* y, int64_t ldy, int64_t by, void* y_bf16, int M, int N, int K, int batch,
+                                      sd_stream_t stream) {
+  SD_REQUIRE(x && w && y && M >= 1 && N >= 1 && K >= 1 && batch >= 1 && batch <= 65535 && ldx >= K && ldy >= N,
+             SD_ERR_INVALID, "sd_matmul_rows_batched: bad argument (M=%d N=%d K=%d batch=%d)", M, N, K, batch);
+  hipStream_t st = (hipStream_t)stream;
+  return w_f32 ? launch_matmul<float>(x, nullptr, ldx, w, nullptr, y, ldy, M, N, K, 0, st, batch, bx, bw, by, (bf16_t*)y_bf16)
+               : launch_matmul<bf16_t>(x, nullptr, ldx, w, nullptr, y, ldy, M, N, K, 1, st, batch, bx, bw, by, (bf16_t*)y_bf16);
 }
 
 extern "C" int sd_rmsnorm_rows(const float* x, const int32_t* rows, const void* w, int w_f32, float offset,
@@ -907,17 +929,69 @@ inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr int kWideRows = 256;  // rows one call of the many-row linear family takes
 struct SeqWs {
   size_t x, h, proj, dec, o, y, mix, ffo, hout, hb, yb, actb, houtb, wide, wide_bytes, attn, attn_bytes, total;
+  // layers normed on their output
+  size_t pq, qe, cqb, conv, step, decay, rlog, sel_e, sel_w, dn, moe, moe_bytes;
 };
+// column offsets inside the fused input projection of a layer normed on its output
+struct PnCols {
+  int dq, dkv, q, k, v, z, xbc, dt, total, inner, conv_ch;
+};
+PnCols pn_cols(const sd_seq_layer& l) {
+  PnCols c = {};
+  int at = 0;
+  if (l.kind == SD_MIX_LATENT) {
+    c.dq = at;  at += l.q_rank;
+    c.dkv = at; at += l.kv_rank + l.rot_dim;
+  } else {
+    c.inner = l.s_heads * l.s_vdim;
+    c.conv_ch = c.inner + 2 * l.s_groups * l.s_state;
+    c.q = at;   at += l.heads * l.dim;
+    c.k = at;   at += l.kv_heads * l.dim;
+    c.v = at;   at += l.kv_heads * l.vdim;
+    c.z = at;   at += c.inner;
+    c.xbc = at; at += c.conv_ch;
+    c.dt = at;  at += l.s_heads;
+  }
+  c.total = at;
+  return c;
+}
 SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
   const int W = m.d.width;
   size_t proj = 0, hk = 0, hv = 0, ff = 0, wide = 0, attn = 0;
+  size_t pq = 0, qe = 0, cq = 0, conv = 0, sh = 0, ne = 0, top = 0, moe = 0;
   const int wr = rows < kWideRows ? rows : kWideRows;
+  auto up = [](size_t& a, size_t b) { a = b > a ? b : a; };
   auto need = [&](const void* tiled, int M, int N, int K) {
     if (!tiled || M <= 16) return;
     const size_t n = sd_linear_wide_workspace_bytes(M, N, K, SD_EPI_F32);
     wide = n > wide ? n : wide;
   };
   for (const sd_seq_layer& l : m.layers) {
+    if (l.block == SD_BLOCK_POSTNORM) {
+      const PnCols c = pn_cols(l);
+      up(proj, (size_t)c.total);
+      need(l.w_in_tiled, wr, c.total, W);
+      need(l.w_o_tiled, wr, W, l.heads * l.vdim);
+      up(hv, (size_t)l.heads * l.vdim);
+      if (l.kind == SD_MIX_LATENT) {
+        up(pq, (size_t)l.heads * (l.dim + l.rot_dim));
+        up(qe, (size_t)l.heads * (l.kv_rank + l.rot_dim));
+        up(cq, (size_t)l.q_rank);
+        up(hv, (size_t)l.heads * l.kv_rank);
+        need(l.w_uq_tiled, wr, l.heads * (l.dim + l.rot_dim), l.q_rank);
+      } else {
+        up(hv, (size_t)c.inner);
+        up(conv, (size_t)c.conv_ch);
+        up(sh, (size_t)l.s_heads);
+        need(l.w_o2_tiled, wr, W, c.inner);
+      }
+      if (l.n_experts > 0) {
+        up(ne, (size_t)l.n_experts);
+        up(top, (size_t)l.top);
+        up(moe, sd_moe_experts_scratch_bytes(rows, l.top, l.n_experts, l.expert_ff, W));
+      }
+      continue;
+    }
     const size_t t = in_cols(l, W).total;
     proj = t > proj ? t : proj;
     const size_t a = (size_t)l.heads * l.dim, b = (size_t)l.heads * l.vdim;
@@ -955,6 +1029,18 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
   w.wide = off; off += al(wide ? wide : 16);
   w.attn_bytes = attn;
   w.attn = off; off += al(attn ? attn : 16);
+  w.pq = off;    off += al(R * pq * f);
+  w.qe = off;    off += al(R * qe * f);
+  w.cqb = off;   off += al(R * cq * 2);
+  w.conv = off;  off += al(R * conv * f);
+  w.step = off;  off += al(R * sh * f);
+  w.decay = off; off += al(R * sh * f);
+  w.rlog = off;  off += al(R * ne * f);
+  w.sel_e = off; off += al(R * top * sizeof(int32_t));
+  w.sel_w = off; off += al(R * top * f);
+  w.dn = off;    off += al(R * top * W * f);
+  w.moe_bytes = moe;
+  w.moe = off;   off += al(moe ? moe : 16);
   w.total = off;
   return w;
 }
@@ -990,6 +1076,26 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
   for (int i = 0; i < desc->n_layers; ++i) {
     const sd_seq_layer& l = m->layers[i];
     const char* bad = nullptr;
+    if (l.block == SD_BLOCK_POSTNORM) {
+      if (l.kind != SD_MIX_LATENT && l.kind != SD_MIX_SOFTMAX_SSD) bad = "a layer normed on its output takes latent attention or attention beside a state-space recurrence";
+      else if (l.heads < 1 || l.dim < 1 || l.vdim < 1 || l.window < 1 || l.keep_first < 0) bad = "head counts / sizes / window";
+      else if (!l.norm_w || !(l.w_in || l.w_in_tiled) || !(l.w_o || l.w_o_tiled) || !l.k_cache) bad = "a null weight or cache";
+      else if ((l.w_in_tiled || l.w_o_tiled || l.w_uq_tiled || l.w_o2_tiled) && desc->weights_f32) bad = "tiled matrices are bf16";
+      else if (l.ff != 0) bad = "a dense feed-forward is not provided for layers normed on their output";
+      else if (l.n_experts > 0 && (l.top < 1 || l.top > l.n_experts || l.expert_ff < 1 || !l.w_router || !l.w_gate_up || !l.w_down_e || !l.norm2_w)) bad = "routed experts need top <= experts, their matrices and norm2";
+      else if (l.kind == SD_MIX_LATENT) {
+        if (l.q_rank < 1 || l.kv_rank < 1 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim || l.rot_dims % 2 ||
+            (l.rot_dims && !l.inv_freq)) bad = "latent ranks / rotary dims";
+        else if (!l.dq_norm_w || !l.dkv_norm_w || !(l.w_uq || l.w_uq_tiled) || !l.w_uk_t || !l.w_uv) bad = "a null latent weight";
+        else if (l.kv_rank > 512) bad = "latent size above 512";
+      } else {
+        if (l.kv_heads < 1 || l.heads % l.kv_heads || l.vdim > 512 || !l.v_cache || !l.q_norm_w || !l.k_norm_w) bad = "attention part";
+        else if (l.s_heads < 1 || l.s_vdim < 1 || l.s_state < 1 || l.s_state > 256 || l.s_groups < 1 || l.s_heads % l.s_groups ||
+                 l.s_taps < 1 || l.s_norm_groups < 1 || (l.s_heads * l.s_vdim) % l.s_norm_groups) bad = "state-space sizes";
+        else if (!l.conv_w || !l.dt_bias || !l.a_log || !l.s_norm_w || !(l.w_o2 || l.w_o2_tiled) || !l.state ||
+                 (l.s_taps > 1 && !l.conv_state)) bad = "a null state-space weight or state";
+      }
+    } else
     if (l.kind != SD_MIX_HEAD_DECAY && l.kind != SD_MIX_CHANNEL_DECAY && l.kind != SD_MIX_WINDOW_POOL) bad = "unknown mixer";
     else if (l.heads < 1 || l.kv_heads < 1 || l.heads % l.kv_heads || l.dim < 1 || l.vdim < 1) bad = "head counts / sizes";
     else if (!l.norm_w || !(l.w_in || l.w_in_tiled) || !(l.w_o || l.w_o_tiled) ||
@@ -1031,6 +1137,106 @@ extern "C" size_t sd_seq_model_workspace_bytes(const sd_seq_model* m, int max_ro
     if (rc__ != SD_OK) return rc__; \
   } while (0)
 
+namespace {
+// One layer normed on its sublayers' outputs: x += norm1(mixer(x)); x += norm2(experts(x)).
+// x [R, W] f32 and its bf16 copy hb are current on entry and on return.
+int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_batch& b, char* base, const SeqWs& w,
+                   sd_stream_t stream) {
+  const sd_seq_model_desc& d = m.d;
+  const int W = d.width, R = b.n_rows, f32 = d.weights_f32, rnd = !f32;
+  const float eps = d.norm_eps;
+  float* x = (float*)(base + w.x);
+  float* proj = (float*)(base + w.proj);
+  float* o = (float*)(base + w.o);
+  float* y = (float*)(base + w.y);
+  float* mix = (float*)(base + w.mix);
+  float* mix2 = (float*)(base + w.ffo);
+  bf16_t* hb = (bf16_t*)(base + w.hb);
+  bf16_t* yb = (bf16_t*)(base + w.yb);
+  void* wide_ws = base + w.wide;
+  const PnCols c = pn_cols(l);
+  const int64_t ld = c.total;
+  const int H = l.heads, dk = l.dim, dv = l.vdim;
+  SQ_TRY(seq_linear(l.w_in, l.w_in_tiled, f32, x, nullptr, W, hb, W, nullptr, proj, ld, R, c.total, W, wide_ws,
+                    w.wide_bytes, stream));
+  if (l.kind == SD_MIX_LATENT) {
+    const int qr = l.q_rank, rk = l.kv_rank, dr = l.rot_dim, dh = dk + dr, de = rk + dr;
+    float* pq = (float*)(base + w.pq);
+    float* qe = (float*)(base + w.qe);
+    bf16_t* cqb = (bf16_t*)(base + w.cqb);
+    // queries: latent, norm, expansion; the rotated part of each head turned
+    SQ_TRY(sd_rmsnorm_parts(proj + c.dq, ld, nullptr, 0, l.dq_norm_w, f32, eps, proj + c.dq, ld,
+                            l.w_uq_tiled ? cqb : nullptr, qr, R, qr, 1, rnd, stream));
+    SQ_TRY(seq_linear(l.w_uq, l.w_uq_tiled, f32, proj + c.dq, nullptr, ld, cqb, qr, nullptr, pq, (int64_t)H * dh, R,
+                      H * dh, qr, wide_ws, w.wide_bytes, stream));
+    // the cached row: normed latent, then the shared rotated key part
+    SQ_TRY(sd_rmsnorm_parts(proj + c.dkv, ld, nullptr, 0, l.dkv_norm_w, f32, eps, proj + c.dkv, ld, nullptr, 0, R, rk,
+                            1, rnd, stream));
+    SQ_TRY(sd_rope_rows(proj + c.dkv + rk, ld, b.row_pos, R, 1, 0, 0, l.rot_dims, 1, l.inv_freq, l.rot_mag, stream));
+    SQ_TRY(sd_cache_append(proj + c.dkv, ld, nullptr, 0, l.k_cache, nullptr, f32, b.row_pos, b.row_slot,
+                           b.block_tables, b.max_blocks, b.page, R, 1, de, 0, stream));
+    // a head's query against the latent: its key expansion, transposed, applied to the unrotated
+    // part; the rotated part is turned into place behind it
+    SQ_TRY(sd_matmul_rows_batched(pq, (int64_t)H * dh, dh, l.w_uk_t, f32, (int64_t)rk * dk, qe, (int64_t)H * de, de,
+                                  nullptr, R, rk, dk, H, stream));
+    if (dr > 0)
+      SQ_TRY(sd_rope_copy_rows(pq, (int64_t)H * dh, dh, dk, qe, (int64_t)H * de, de, rk, b.row_pos, R, H, dr,
+                               l.rot_dims, 1, l.inv_freq, l.rot_mag, stream));
+    SQ_TRY(sd_window_softmax_attention(qe, (int64_t)H * de, l.k_cache, nullptr, f32, b.row_pos, b.row_slot,
+                                       b.block_tables, b.max_blocks, b.page, R, H, 1, de, rk, l.window, 0,
+                                       l.score_scale, o, nullptr, stream));
+    // a head's value expansion applied to its weighted latent
+    SQ_TRY(sd_matmul_rows_batched(o, (int64_t)H * rk, rk, l.w_uv, f32, (int64_t)dv * rk, y, (int64_t)H * dv, dv,
+                                  l.w_o_tiled ? yb : nullptr, R, dv, rk, H, stream));
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, y, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
+                      H * dv, wide_ws, w.wide_bytes, stream));
+    SQ_TRY(sd_postnorm_residual(x, mix, 1, 1.f, nullptr, 0.f, l.norm_w, f32, eps, hb, R, W, stream));
+  } else {
+    const int G = l.kv_heads;
+    // attention: q and k normed over the whole projection, no rotation
+    SQ_TRY(sd_rmsnorm_parts(proj + c.q, ld, nullptr, 0, l.q_norm_w, f32, eps, proj + c.q, ld, nullptr, 0, R, H * dk, 1,
+                            0, stream));
+    SQ_TRY(sd_rmsnorm_parts(proj + c.k, ld, nullptr, 0, l.k_norm_w, f32, eps, proj + c.k, ld, nullptr, 0, R, G * dk, 1,
+                            0, stream));
+    SQ_TRY(sd_cache_append(proj + c.k, ld, proj + c.v, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
+                           b.block_tables, b.max_blocks, b.page, R, G, dk, dv, stream));
+    SQ_TRY(sd_window_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
+                                       b.block_tables, b.max_blocks, b.page, R, H, G, dk, dv, l.window, l.keep_first,
+                                       l.score_scale, o, l.w_o_tiled ? yb : nullptr, stream));
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, o, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
+                      H * dv, wide_ws, w.wide_bytes, stream));
+    // state-space recurrence: convolution + silu over x, B, C; step sizes; scan; gate, group norm
+    float* conv = (float*)(base + w.conv);
+    float* step = (float*)(base + w.step);
+    float* decay = (float*)(base + w.decay);
+    const int Hs = l.s_heads, P = l.s_vdim, N = l.s_state, Gs = l.s_groups, inner = c.inner;
+    SQ_TRY(sd_causal_conv_rows(proj + c.xbc, ld, l.conv_w, l.conv_b, f32, l.conv_state, b.row_pos, b.row_slot,
+                               b.entries, b.n_entries, conv, c.conv_ch, R, c.conv_ch, l.s_taps, 1, stream));
+    SQ_TRY(sd_ssd_steps(proj + c.dt, ld, l.dt_bias, l.a_log, f32, step, decay, R, Hs, stream));
+    SQ_TRY(sd_decay_scan_rows(conv + inner + Gs * N, conv + inner, c.conv_ch, conv, c.conv_ch, decay, step, l.skip_d,
+                              f32, l.state, b.entries, b.n_entries, o, Hs, Gs, N, P, stream));
+    SQ_TRY(sd_rmsnorm_parts(o, inner, proj + c.z, ld, l.s_norm_w, f32, eps, y, inner, l.w_o2_tiled ? yb : nullptr,
+                            inner, R, inner, l.s_norm_groups, rnd, stream));
+    SQ_TRY(seq_linear(l.w_o2, l.w_o2_tiled, f32, y, nullptr, inner, yb, inner, nullptr, mix2, W, R, W, inner, wide_ws,
+                      w.wide_bytes, stream));
+    SQ_TRY(sd_postnorm_residual(x, mix, 1, l.left_scale, mix2, l.right_scale, l.norm_w, f32, eps, hb, R, W, stream));
+  }
+  if (l.n_experts > 0) {
+    float* rlog = (float*)(base + w.rlog);
+    int32_t* sel_e = (int32_t*)(base + w.sel_e);
+    float* sel_w = (float*)(base + w.sel_w);
+    float* dn = (float*)(base + w.dn);
+    const int E = l.n_experts;
+    SQ_TRY(sd_matmul_rows(x, nullptr, W, l.w_router, f32, nullptr, rlog, E, R, E, W, stream));
+    SQ_TRY(sd_moe_route(rlog, E, sel_e, sel_w, R, E, l.top, 0, 0, stream));
+    SQ_TRY(sd_moe_experts(x, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, E, l.expert_ff, W, 1, 0,
+                          base + w.moe, w.moe_bytes, stream));
+    SQ_TRY(sd_postnorm_residual(x, dn, l.top, 1.f, nullptr, 0.f, l.norm2_w, f32, eps, hb, R, W, stream));
+  }
+  return SD_OK;
+}
+}  // namespace
+
 extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void* workspace,
                                     size_t workspace_bytes, sd_stream_t stream) {
   SD_REQUIRE(m && b && workspace, SD_ERR_INVALID, "sd_seq_model_forward: null argument");
@@ -1062,12 +1268,31 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
   bf16_t* houtb = (bf16_t*)(base + w.houtb);
   void* wide_ws = base + w.wide;
 
-  if (f32) embed_rows_kernel<float><<<R, 256, 0, st>>>(b->tokens, (const float*)d.embed, x, W, d.vocab);
-  else embed_rows_kernel<bf16_t><<<R, 256, 0, st>>>(b->tokens, (const bf16_t*)d.embed, x, W, d.vocab);
-  SD_CHECK_LAUNCH("sd_seq_model_forward (embed)");
+  const bool hashed = d.bigram || (d.embed_scale != 0.f && d.embed_scale != 1.f) || m->layers[0].block == SD_BLOCK_POSTNORM;
+  if (hashed) {
+    SD_REQUIRE(!d.bigram || b->prev_tokens, SD_ERR_INVALID, "sd_seq_model_forward: a bigram table needs prev_tokens");
+    SQ_TRY(sd_embed_hashed(b->tokens, b->prev_tokens, d.embed, d.bigram, f32, d.embed_scale != 0.f ? d.embed_scale : 1.f,
+                           d.buckets, d.mul_prev, d.mul_cur, x, hb, R, W, d.vocab, stream));
+  } else {
+    if (f32) embed_rows_kernel<float><<<R, 256, 0, st>>>(b->tokens, (const float*)d.embed, x, W, d.vocab);
+    else embed_rows_kernel<bf16_t><<<R, 256, 0, st>>>(b->tokens, (const bf16_t*)d.embed, x, W, d.vocab);
+    SD_CHECK_LAUNCH("sd_seq_model_forward (embed)");
+  }
 
   for (int li = 0; li < d.n_layers; ++li) {
     const sd_seq_layer& l = m->layers[li];
+    if (l.block == SD_BLOCK_POSTNORM) {
+      SQ_TRY(postnorm_layer(*m, l, *b, base, w, stream));
+      if (b->layer_out) {
+        const hipError_t e = hipMemcpyAsync(b->layer_out + (size_t)li * R * W, x, (size_t)R * W * sizeof(float),
+                                            hipMemcpyDeviceToDevice, st);
+        SD_REQUIRE(e == hipSuccess, SD_ERR_HIP, "sd_seq_model_forward: copying a layer's output: %s",
+                   hipGetErrorString(e));
+      }
+      continue;
+    }
+    SD_REQUIRE(li == 0 || m->layers[li - 1].block != SD_BLOCK_POSTNORM, SD_ERR_UNSUPPORTED,
+               "sd_seq_model_forward: a gated layer after a layer normed on its output is not provided");
     const InCols c = in_cols(l, W);
     const int64_t ld = c.total;
     const int H = l.heads, G = l.kv_heads, dk = l.dim, dv = l.vdim;
@@ -1127,10 +1352,12 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
     }
   }
   if (b->n_out > 0) {
-    SQ_TRY(sd_rmsnorm_rows(x, b->out_rows, d.final_norm_w, f32, 1.f, d.norm_eps, hout,
+    SQ_TRY(sd_rmsnorm_rows(x, b->out_rows, d.final_norm_w, f32, d.plain_norm ? 0.f : 1.f, d.norm_eps, hout,
                            d.head_tiled ? houtb : nullptr, b->n_out, W, stream));
-    SQ_TRY(seq_linear(d.embed, d.head_tiled, f32, hout, nullptr, W, houtb, W, nullptr, b->logits, d.vocab, b->n_out,
-                      d.vocab, W, wide_ws, w.wide_bytes, stream));
+    SQ_TRY(seq_linear(d.head ? d.head : d.embed, d.head_tiled, f32, hout, nullptr, W, houtb, W, nullptr, b->logits,
+                      d.vocab, b->n_out, d.vocab, W, wide_ws, w.wide_bytes, stream));
+    if (d.logit_scale != 0.f && d.logit_scale != 1.f)
+      SQ_TRY(sd_scale_rows(b->logits, d.vocab, d.logit_scale, b->n_out, d.vocab, stream));
   }
   return SD_OK;
 }

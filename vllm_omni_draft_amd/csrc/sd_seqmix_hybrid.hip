@@ -1,0 +1,1066 @@
+// Mechanisms of hybrid decoders (layer-list models whose sublayers are normed on their output):
+// softmax attention over a sliding window with kept first tokens, also over latent rows that
+// serve as key and value at once; rotary turns of a sub-vector with a magnitude factor; a causal
+// convolution with a carried tail; the step sizes of a state-space recurrence; routed experts
+// grouped by expert on the device; the residual update with a norm on the sublayer's output.
+//
+// Arithmetic as in sd_seqmix.hip: activations are f32 buffers, scores, softmax weights, norms,
+// router scores, step sizes and decays are f32 always; with bf16 weights the operands of matrix
+// products are rounded to bf16 values where they are produced and the cache holds bf16.  Every
+// output element is summed in an order fixed by the token's own position in its sequence.
+#include <math.h>
+
+#include "sd_common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld_f(const T* p);
+template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return (float)*p; }
+template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
+template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = (bf16_t)v; }
+
+__device__ __forceinline__ float maybe_round(float v, int round) { return round ? round_bf16(v) : v; }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z * sigmoid_f(z); }
+
+// Sum over a workgroup of up to 256 threads in a fixed order (waves' sums in wave order).
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int w = 1; w < n_waves; ++w) s += red[w];
+  return s;
+}
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_hashed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ prev,
+                                    const T* __restrict__ table, const T* __restrict__ bigram, float scale,
+                                    int buckets, int mul_prev, int mul_cur, float* __restrict__ x,
+                                    bf16_t* __restrict__ x_b, int W, int vocab) {
+  const int r = blockIdx.x;
+  int tok = tokens[r];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  long long brow = -1;
+  if (bigram) {
+    const int p = prev ? prev[r] : -1;
+    brow = p < 0 ? (long long)buckets
+                 : (long long)(((long long)p * mul_prev + (long long)tokens[r] * mul_cur) % buckets);
+    if (brow < 0) brow += buckets;
+  }
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = ld_f(table + (size_t)tok * W + c) * scale;
+    if (brow >= 0) v += ld_f(bigram + (size_t)brow * W + c);
+    x[(size_t)r * W + c] = v;
+    if (x_b) x_b[(size_t)r * W + c] = (bf16_t)v;
+  }
+}
+
+// ------------------------------------------------------------------ norm over parts of a row
+// One workgroup per (row, part).
+template <typename T>
+__global__ void rmsnorm_parts_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ gate,
+                                     int64_t ldg, const T* __restrict__ w, float eps, float* __restrict__ out,
+                                     int64_t ldo, bf16_t* __restrict__ out_b, int64_t ldob, int pw, int round) {
+  __shared__ float red[4];
+  const int r = blockIdx.x, c0 = blockIdx.y * pw;
+  const float* xr = x + (size_t)r * ldx + c0;
+  const float* gr = gate ? gate + (size_t)r * ldg + c0 : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < pw; c += blockDim.x) {
+    const float v = gr ? xr[c] * silu_f(gr[c]) : xr[c];
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)pw + eps);
+  for (int c = threadIdx.x; c < pw; c += blockDim.x) {
+    float v = gr ? xr[c] * silu_f(gr[c]) : xr[c];
+    v *= rstd;
+    if (w) v *= ld_f(w + c0 + c);
+    v = maybe_round(v, round);
+    out[(size_t)r * ldo + c0 + c] = v;
+    if (out_b) out_b[(size_t)r * ldob + c0 + c] = (bf16_t)v;
+  }
+}
+
+// ------------------------------------------------------------------ rotary turn of a sub-vector
+// One wave per (row, head): n channels from src to dst (the same place or another), the first
+// `dims` of them turned; the angle is formed in f64 (position times frequency).
+__global__ void rope_copy_kernel(const float* __restrict__ src, int64_t lds_, int src_hs, int src_off,
+                                 float* __restrict__ dst, int64_t ldd, int dst_hs, int dst_off,
+                                 const int32_t* __restrict__ row_pos, int n, int dims, int layout,
+                                 const double* __restrict__ inv_freq, float mag) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const float* in = src + (size_t)r * lds_ + (size_t)h * src_hs + src_off;
+  float* out = dst + (size_t)r * ldd + (size_t)h * dst_hs + dst_off;
+  const int pos = row_pos[r];
+  for (int i = threadIdx.x; i < dims / 2; i += blockDim.x) {
+    const double a = (double)pos * inv_freq[i];
+    const float cs = (float)cos(a) * mag, sn = (float)sin(a) * mag;
+    const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
+    const float u = in[iu], v = in[iv];
+    out[iu] = u * cs - v * sn;
+    out[iv] = v * cs + u * sn;
+  }
+  if (in != out)
+    for (int c = dims + threadIdx.x; c < n; c += blockDim.x) out[c] = in[c];
+}
+
+// ------------------------------------------------------------------ cache append
+template <typename T>
+__global__ void cache_append_kernel(const float* __restrict__ k, int64_t ldk, const float* __restrict__ v,
+                                    int64_t ldv, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                                    const int32_t* __restrict__ block_tables, int max_blocks, int page, int G,
+                                    int dk, int dv) {
+  const int r = blockIdx.x, g = blockIdx.y;
+  const int pos = row_pos[r];
+  const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+  const size_t at = ((size_t)pg * G + g) * page + pos % page;
+  for (int c = threadIdx.x; c < dk; c += blockDim.x) st_f(k_cache + at * dk + c, k[(size_t)r * ldk + (size_t)g * dk + c]);
+  if (v)
+    for (int c = threadIdx.x; c < dv; c += blockDim.x) st_f(v_cache + at * dv + c, v[(size_t)r * ldv + (size_t)g * dv + c]);
+}
+
+// ------------------------------------------------------------------ softmax window attention
+constexpr int kTile = 256;     // keys per tile
+constexpr int kLoads = 16;     // 16-byte pieces of a key row a thread has in flight
+
+template <typename T> struct Piece;
+template <> struct Piece<bf16_t> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& raw, float* f) {
+    const bf16x8 v = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+  }
+};
+template <> struct Piece<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void unpack(const u32x4& raw, float* f) {
+    const f32x4 v = __builtin_bit_cast(f32x4, raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = v[i];
+  }
+};
+
+// s[hq] += q[hq] . k, channels ascending.  vec: rows are 16-byte aligned and dk a multiple of the
+// piece size; then up to kLoads pieces are asked for before the first is used.
+template <typename KT, int NH>
+__device__ __forceinline__ void score_key(const KT* __restrict__ kr, const float* __restrict__ qs, int dk, int nh,
+                                          bool vec, float* s) {
+  constexpr int E = Piece<KT>::E;
+  if (vec) {
+    for (int c = 0; c < dk; c += kLoads * E) {
+      u32x4 raw[kLoads];
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) {   // unguarded, on an address clamped into the row
+        const int ci = c + i * E < dk ? c + i * E : dk - E;
+        raw[i] = *reinterpret_cast<const u32x4*>(kr + ci);
+      }
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) {
+        if (c + i * E < dk) {
+          float kf[E];
+          Piece<KT>::unpack(raw[i], kf);
+#pragma unroll
+          for (int hq = 0; hq < NH; ++hq)
+            if (hq < nh) {
+#pragma unroll
+              for (int e = 0; e < E; ++e) s[hq] = fmaf(qs[hq * dk + c + i * E + e], kf[e], s[hq]);
+            }
+        }
+      }
+    }
+    return;
+  }
+  for (int c = 0; c < dk; ++c) {
+    const float kf = ld_f(kr + c);
+#pragma unroll
+    for (int hq = 0; hq < NH; ++hq)
+      if (hq < nh) s[hq] = fmaf(qs[hq * dk + c], kf, s[hq]);
+  }
+}
+
+// One workgroup per (row, kv head, group of up to NH query heads of that kv head).  Per tile of
+// 256 keys: a thread per key scores it against the query heads (q in LDS); the tile's maximum
+// moves the running maximum and rescales what has been summed; then a wave per key, lanes over
+// value columns, adds the weighted value rows.  NC: value columns per lane (dv <= 64 * NC).
+template <typename T, int NH, int NC>
+__global__ __launch_bounds__(256) void window_softmax_attn_kernel(
+    const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    int v_row, const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+    const int32_t* __restrict__ block_tables, int max_blocks, int page, int H, int G, int dk, int dv, int window,
+    int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups) {
+  extern __shared__ float lds[];
+  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [kTile] cache row of the key
+  float* wt = reinterpret_cast<float*>(vat + kTile);                     // [NH][kTile]
+  float* qs = wt + NH * kTile;                                           // [NH][dk]
+  float* m_run = qs + NH * dk;                                           // [NH] running maximum
+  float* l_run = m_run + NH;                                             // [NH] running sum
+  float* corr = l_run + NH;                                              // [NH]
+  float* red = corr + NH;                                                // [4][dv]
+  const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+  const int hgroup = blockIdx.z;
+  const int qh = H / G;
+  const int h0 = g * qh + hgroup * NH;
+  const int nh = qh - hgroup * NH < NH ? qh - hgroup * NH : NH;
+  const int i = row_pos[r];
+  const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
+  for (int c = tid; c < nh * dk; c += 256) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
+  if (tid < NH) {
+    m_run[tid] = -INFINITY;
+    l_run[tid] = 0.f;
+  }
+  const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
+  const int n_kept = keep_first < t_first ? keep_first : t_first;   // kept tokens that left the window
+  const int total = n_kept + (i - t_first + 1);
+  const bool vec = dk % Piece<T>::E == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
+  const int wave = tid >> 6, lane = tid & 63;
+  float acc[NH][NC];
+#pragma unroll
+  for (int hq = 0; hq < NH; ++hq)
+#pragma unroll
+    for (int m = 0; m < NC; ++m) acc[hq][m] = 0.f;
+  __syncthreads();
+  for (int base = 0; base < total; base += kTile) {
+    const int idx = base + tid;
+    {
+      float s[NH];
+#pragma unroll
+      for (int hq = 0; hq < NH; ++hq) s[hq] = 0.f;
+      if (idx < total) {
+        const int j = idx < n_kept ? idx : t_first + (idx - n_kept);
+        const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
+        score_key<T, NH>(k_cache + at * dk, qs, dk, nh, vec, s);
+        vat[tid] = at;
+      }
+#pragma unroll
+      for (int hq = 0; hq < NH; ++hq)
+        if (hq < nh) wt[hq * kTile + tid] = idx < total ? s[hq] * scale : -INFINITY;
+    }
+    __syncthreads();
+    for (int hq = wave; hq < nh; hq += 4) {      // the tile's maximum per head, a wave per head
+      float m = fmaxf(fmaxf(wt[hq * kTile + lane], wt[hq * kTile + 64 + lane]),
+                      fmaxf(wt[hq * kTile + 128 + lane], wt[hq * kTile + 192 + lane]));
+      m = wave_max(m);
+      if (lane == 0) {
+        const float m_old = m_run[hq], m_new = fmaxf(m_old, m);
+        corr[hq] = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        m_run[hq] = m_new;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int hq = 0; hq < NH; ++hq)
+      if (hq < nh) {
+        const float sv = wt[hq * kTile + tid];
+        wt[hq * kTile + tid] = idx < total ? expf(sv - m_run[hq]) : 0.f;
+      }
+    __syncthreads();
+    for (int hq = wave; hq < nh; hq += 4) {      // running sum of the weights
+      float sum = (wt[hq * kTile + lane] + wt[hq * kTile + 64 + lane]) +
+                  (wt[hq * kTile + 128 + lane] + wt[hq * kTile + 192 + lane]);
+      sum = wave_sum(sum);
+      if (lane == 0) l_run[hq] = l_run[hq] * corr[hq] + sum;
+    }
+#pragma unroll
+    for (int hq = 0; hq < NH; ++hq)
+      if (hq < nh) {
+        const float cf = corr[hq];
+#pragma unroll
+        for (int m = 0; m < NC; ++m) acc[hq][m] *= cf;
+      }
+    const int n_here = total - base < kTile ? total - base : kTile;
+    constexpr int kBatch = NC <= 2 ? 16 : (NC <= 4 ? 8 : 4);   // value rows a wave has in flight
+    for (int kk0 = wave; kk0 < n_here; kk0 += 4 * kBatch) {
+      float vf[kBatch][NC];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int kk = kk0 + 4 * u < n_here ? kk0 + 4 * u : n_here - 1;
+        const size_t at = vat[kk];
+#pragma unroll
+        for (int m = 0; m < NC; ++m)
+          vf[u][m] = ld_f(v_cache + at * v_row + (lane + 64 * m < dv ? lane + 64 * m : dv - 1));
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int kk = kk0 + 4 * u;
+        if (kk < n_here) {
+#pragma unroll
+          for (int hq = 0; hq < NH; ++hq)
+            if (hq < nh) {
+              const float w = wt[hq * kTile + kk];
+#pragma unroll
+              for (int m = 0; m < NC; ++m) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
+            }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // the four waves' sums in wave order, one head at a time
+#pragma unroll
+  for (int hq = 0; hq < NH; ++hq) {
+    if (hq < nh) {
+#pragma unroll
+      for (int m = 0; m < NC; ++m)
+        if (lane + 64 * m < dv) red[wave * dv + lane + 64 * m] = acc[hq][m];
+      __syncthreads();
+      const float inv = 1.f / l_run[hq];
+      for (int c = tid; c < dv; c += 256) {
+        const float o = (((red[c] + red[dv + c]) + red[2 * dv + c]) + red[3 * dv + c]) * inv;
+        const size_t at = (size_t)r * H * dv + (size_t)(h0 + hq) * dv + c;
+        out[at] = o;
+        if (out_b) out_b[at] = (bf16_t)o;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+template <typename T, int NH>
+void launch_softmax_nc(dim3 grid, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq, const void* kc,
+                       const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot, const int32_t* bt,
+                       int max_blocks, int page, int H, int G, int dk, int dv, int window, int keep_first, float scale,
+                       float* out, bf16_t* out_b, int n_hgroups) {
+#define SD_GO(NC)                                                                                                  \
+  window_softmax_attn_kernel<T, NH, NC><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
+                                                                row_slot, bt, max_blocks, page, H, G, dk, dv, window, \
+                                                                keep_first, scale, out, out_b, n_hgroups)
+  if (nc == 1) SD_GO(1);
+  else if (nc == 2) SD_GO(2);
+  else if (nc == 4) SD_GO(4);
+  else SD_GO(8);
+#undef SD_GO
+}
+
+// ------------------------------------------------------------------ causal convolution
+// out[r, c] = act(b[c] + sum_j w[c, taps-1-j] * in(r, j)).  One workgroup per (row, 256 channels).
+template <typename T>
+__global__ void causal_conv_rows_kernel(const float* __restrict__ x, int64_t ldx, const T* __restrict__ w,
+                                        const T* __restrict__ b, const float* __restrict__ conv_state,
+                                        const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                                        float* __restrict__ out, int64_t ldo, int C, int taps, int act) {
+  const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int slot = row_slot[r], pos = row_pos[r];
+  int t = 0;   // rows of this entry before r, as far as the taps reach
+  while (t < taps - 1 && r - t - 1 >= 0 && row_slot[r - t - 1] == slot) ++t;
+  float acc = b ? ld_f(b + c) : 0.f;
+  // oldest input first, so that the sum's order is that of a plain convolution
+  for (int j = taps - 1; j >= 0; --j) {
+    float in = 0.f;
+    if (j <= t) in = x[(size_t)(r - j) * ldx + c];
+    else if (pos - j >= 0) in = conv_state[((size_t)slot * (taps - 1) + (taps - 1 - (j - t))) * C + c];
+    acc = fmaf(ld_f(w + (size_t)c * taps + (taps - 1 - j)), in, acc);
+  }
+  out[(size_t)r * ldo + c] = act ? silu_f(acc) : acc;
+}
+
+// The entry's last taps-1 inputs become the slot's state (oldest first).  One thread per channel.
+__global__ void conv_state_update_kernel(const float* __restrict__ x, int64_t ldx, float* __restrict__ conv_state,
+                                         const int32_t* __restrict__ entries, int C, int taps) {
+  const int e = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int slot = entries[4 * e], row0 = entries[4 * e + 1], len = entries[4 * e + 2], pos0 = entries[4 * e + 3];
+  float* st = conv_state + (size_t)slot * (taps - 1) * C + c;
+  for (int s = 0; s < taps - 1; ++s) {   // ascending: an old element is read before its place is written
+    const int at = len + s - (taps - 1);  // index among the entry's inputs, negative: before the entry
+    float v;
+    if (at >= 0) v = x[(size_t)(row0 + at) * ldx + c];
+    else v = pos0 + at >= 0 ? st[(size_t)(len + s) * C] : 0.f;
+    st[(size_t)s * C] = v;
+  }
+}
+
+template <typename T>
+__global__ void ssd_steps_kernel(const float* __restrict__ dt, int64_t ld, const T* __restrict__ dt_bias,
+                                 const T* __restrict__ a_log, float* __restrict__ step, float* __restrict__ decay,
+                                 int n, int H) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int r = i / H, h = i % H;
+  const float z = dt[(size_t)r * ld + h] + ld_f(dt_bias + h);
+  const float sp = z > 20.f ? z : log1pf(expf(z));
+  step[i] = sp;
+  decay[i] = expf(-expf(ld_f(a_log + h)) * sp);
+}
+
+// ------------------------------------------------------------------ scan with a decay per (row, head)
+constexpr int kStrip = 16;
+constexpr int kScanLoads = 8;
+constexpr int kScanLoadsV = 16;
+constexpr int kScanChunk = 16;
+// S <- d_t S + (a_t k_t) v_t^T, o_t = S^T q_t + skip v_t.  A thread owns 16 consecutive key channels
+// of one value column; strips' partial dot products are added in strip order (the skip term rides
+// on strip 0).  Chunks of tokens go global -> registers -> LDS with the next chunk's loads in flight.
+template <typename T>
+__global__ __launch_bounds__(256) void decay_scan_rows_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, int64_t ldqk, const float* __restrict__ v, int64_t ldv,
+    const float* __restrict__ decay, const float* __restrict__ k_scale, const T* __restrict__ skip,
+    float* __restrict__ state, const int32_t* __restrict__ entries,
+    float* __restrict__ out, int H, int hpg, int dk, int dv, int CT, int NS, int CH) {
+  extern __shared__ float lds[];
+  const int dkp = NS * kStrip;
+  float* qs = lds;                  // [CH][dkp]
+  float* ks = qs + CH * dkp;        // [CH][dkp]
+  float* vs = ks + CH * dkp;        // [CH][CT]
+  float* dsc = vs + CH * CT;        // [CH] decay
+  float* asc = dsc + CH;            // [CH] key scale
+  float* part = asc + CH;           // [CH][NS][CT]
+  const int tid = threadIdx.x, nthr = CT * NS;
+  const int c = tid % CT, s = tid / CT;
+  const int h = blockIdx.y, e = blockIdx.z;
+  const int gq = h / hpg;
+  const int col = blockIdx.x * CT + c;
+  const int slot = entries[4 * e], row0 = entries[4 * e + 1], len = entries[4 * e + 2], pos0 = entries[4 * e + 3];
+  float* st = state + ((size_t)slot * H + h) * dk * dv;
+  const int r0 = s * kStrip;
+  float S[kStrip];
+#pragma unroll
+  for (int r = 0; r < kStrip; ++r)
+    S[r] = (pos0 > 0 && r0 + r < dk && col < dv) ? st[(size_t)(r0 + r) * dv + col] : 0.f;
+  const float skip_h = skip ? ld_f(skip + h) : 0.f;
+  float pq[kScanLoads], pk[kScanLoads], pv[kScanLoadsV], pd = 0.f, pa = 1.f;
+  auto fetch = [&](int t0) {
+    const int nt = len - t0 < CH ? len - t0 : CH;
+#pragma unroll
+    for (int i = 0; i < kScanLoads; ++i) {
+      const int idx = tid + i * nthr;
+      const int t = idx / dkp, ch = idx % dkp;
+      const bool in = idx < nt * dkp && ch < dk;
+      const int tc = t < nt ? t : nt - 1, cc = ch < dk ? ch : dk - 1;
+      const size_t at = (size_t)(row0 + t0 + tc) * ldqk + (size_t)gq * dk + cc;
+      const float lq = q[at], lk = k[at];
+      pq[i] = in ? lq : 0.f;
+      pk[i] = in ? lk : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < kScanLoadsV; ++i) {
+      const int idx = tid + i * nthr;
+      const int t = idx / CT, vcol = blockIdx.x * CT + idx % CT;
+      const bool in = idx < nt * CT && vcol < dv;
+      const int tc = t < nt ? t : nt - 1, vc2 = vcol < dv ? vcol : dv - 1;
+      const float lv = v[(size_t)(row0 + t0 + tc) * ldv + (size_t)h * dv + vc2];
+      pv[i] = in ? lv : 0.f;
+    }
+    {
+      const int tc = tid < nt ? tid : nt - 1;
+      pd = decay[(size_t)(row0 + t0 + tc) * H + h];
+      pa = k_scale ? k_scale[(size_t)(row0 + t0 + tc) * H + h] : 1.f;
+    }
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < len; t0 += CH) {
+    const int nt = len - t0 < CH ? len - t0 : CH;
+#pragma unroll
+    for (int i = 0; i < kScanLoads; ++i) {
+      const int idx = tid + i * nthr;
+      if (idx < CH * dkp) {
+        qs[idx] = pq[i];
+        ks[idx] = pk[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kScanLoadsV; ++i) {
+      const int idx = tid + i * nthr;
+      if (idx < CH * CT) vs[idx] = pv[i];
+    }
+    if (tid < CH) {
+      dsc[tid] = pd;
+      asc[tid] = pa;
+    }
+    __syncthreads();
+    if (t0 + CH < len) fetch(t0 + CH);
+    for (int t = 0; t < nt; ++t) {
+      const float vv = vs[t * CT + c];
+      const float d = dsc[t], av = asc[t] * vv;
+      const float* qt = qs + t * dkp + r0;
+      const float* kt = ks + t * dkp + r0;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < kStrip; ++r) {
+        S[r] = fmaf(d, S[r], kt[r] * av);
+        acc = fmaf(S[r], qt[r], acc);
+      }
+      if (s == 0) acc = fmaf(skip_h, vv, acc);
+      part[(t * NS + s) * CT + c] = acc;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nt * CT; idx += nthr) {
+      const int t = idx / CT, cc = idx % CT;
+      const int ocol = blockIdx.x * CT + cc;
+      if (ocol >= dv) continue;
+      float o = part[(t * NS) * CT + cc];
+      for (int ss = 1; ss < NS; ++ss) o += part[(t * NS + ss) * CT + cc];
+      out[(size_t)(row0 + t0 + t) * ((size_t)H * dv) + (size_t)h * dv + ocol] = o;
+    }
+  }
+  if (col < dv) {
+#pragma unroll
+    for (int r = 0; r < kStrip; ++r)
+      if (r0 + r < dk) st[(size_t)(r0 + r) * dv + col] = S[r];
+  }
+}
+
+// ------------------------------------------------------------------ routed experts
+// One wave per row: scores, then `top` rounds of a wave-wide arg-max (lowest index among equals).
+__global__ void moe_route_kernel(const float* __restrict__ logits, int64_t ld, int32_t* __restrict__ sel_e,
+                                 float* __restrict__ sel_w, int E, int top, int score_kind, int renorm) {
+  extern __shared__ float sc[];   // [E]
+  const int r = blockIdx.x, lane = threadIdx.x;
+  const float* z = logits + (size_t)r * ld;
+  if (score_kind == 0) {
+    for (int e = lane; e < E; e += 64) sc[e] = sigmoid_f(z[e]);
+  } else {
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, z[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float p = expf(z[e] - m);
+      sc[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) sc[e] /= sum;
+  }
+  __syncthreads();
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = sc[e];
+      if (v > best) {   // (ascending e: the first of equals stays)
+        best = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+      }
+    }
+    if (lane == 0) {
+      sel_e[(size_t)r * top + j] = bi;
+      sel_w[(size_t)r * top + j] = best;
+      sc[bi] = -INFINITY;
+    }
+    total += best;
+    __syncthreads();
+  }
+  if (renorm && lane == 0)
+    for (int j = 0; j < top; ++j) sel_w[(size_t)r * top + j] /= total;
+}
+
+constexpr int kMoeBM = 32;   // assignment rows per tile of the grouped products
+// cnt[e] = assignments of expert e.  One workgroup per expert.
+__global__ void moe_count_kernel(const int32_t* __restrict__ sel_e, int n, int32_t* __restrict__ cnt) {
+  __shared__ float red[4];
+  const int e = blockIdx.x;
+  float c = 0.f;
+  for (int a = threadIdx.x; a < n; a += blockDim.x) c += sel_e[a] == e ? 1.f : 0.f;
+  c = block_sum(c, red);
+  if (threadIdx.x == 0) cnt[e] = (int)c;
+}
+// perm: assignments grouped by expert, ascending inside a group; tiles[t] = {expert, first index
+// in perm, rows}; n_tiles[0] = number of tiles.  One workgroup of 256 per expert.
+__global__ void moe_group_kernel(const int32_t* __restrict__ sel_e, int n, const int32_t* __restrict__ cnt, int E,
+                                 int32_t* __restrict__ perm, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles) {
+  __shared__ int wsum[4];
+  __shared__ int base_s;
+  const int e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  int off = 0, toff = 0;
+  for (int i = 0; i < e; ++i) {
+    off += cnt[i];
+    toff += (cnt[i] + kMoeBM - 1) / kMoeBM;
+  }
+  const int mine = cnt[e];
+  const int my_tiles = (mine + kMoeBM - 1) / kMoeBM;
+  for (int t = tid; t < my_tiles; t += 256) {
+    tiles[3 * (toff + t)] = e;
+    tiles[3 * (toff + t) + 1] = off + t * kMoeBM;
+    tiles[3 * (toff + t) + 2] = mine - t * kMoeBM < kMoeBM ? mine - t * kMoeBM : kMoeBM;
+  }
+  if (e == E - 1 && tid == 0) n_tiles[0] = toff + my_tiles;
+  if (tid == 0) base_s = 0;
+  __syncthreads();
+  for (int a0 = 0; a0 < n; a0 += 256) {
+    const int a = a0 + tid;
+    const bool hit = a < n && sel_e[a] == e;
+    const unsigned long long bal = __ballot(hit);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int wbase = base_s;
+    for (int w = 0; w < wave; ++w) wbase += wsum[w];
+    if (hit) perm[off + wbase + before] = a;
+    __syncthreads();
+    if (tid == 0) base_s += wsum[0] + wsum[1] + wsum[2] + wsum[3];
+    __syncthreads();
+  }
+}
+
+// act[a, n] = silu(s * (gate_e x)) * (s * (up_e x)) for the assignments of one tile (s = weight of
+// the assignment when scale_input, else 1).  Each output is summed over k ascending.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(
+    const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const T* __restrict__ Wgu,
+    float* __restrict__ act, int top, int F, int K, int scale_input, int round) {
+  constexpr int BM = kMoeBM, BN = 64, BK = 16, TM = 2, TN = 4;
+  if ((int)blockIdx.y >= n_tiles[0]) return;
+  __shared__ float xs[BK][BM + 1];
+  __shared__ float wg[BK][BN + 1];
+  __shared__ float wu[BK][BN + 1];
+  __shared__ int arow[BM];
+  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  const int tid = threadIdx.x, tx = tid % (BN / TN), ty = tid / (BN / TN);
+  const int n0 = blockIdx.x * BN;
+  const T* Wg = Wgu + (size_t)e * 2 * F * K;
+  const T* Wu = Wg + (size_t)F * K;
+  if (tid < BM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  __syncthreads();
+  float ag[TM][TN], au[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) ag[i][j] = au[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int idx = tid; idx < BM * BK; idx += 256) {
+      const int m = idx / BK, kk = idx % BK;
+      const int a = arow[m];
+      xs[kk][m] = (a >= 0 && k0 + kk < K) ? maybe_round(X[(size_t)(a / top) * ldx + k0 + kk], round) : 0.f;
+    }
+    for (int idx = tid; idx < BN * BK; idx += 256) {
+      const int n = idx / BK, kk = idx % BK;
+      const bool in = n0 + n < F && k0 + kk < K;
+      wg[kk][n] = in ? ld_f(Wg + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
+      wu[kk][n] = in ? ld_f(Wu + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[TM], bg[TN], bu[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = xs[kk][ty * TM + i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        bg[j] = wg[kk][tx * TN + j];
+        bu[j] = wu[kk][tx * TN + j];
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          ag[i][j] = fmaf(a[i], bg[j], ag[i][j]);
+          au[i][j] = fmaf(a[i], bu[j], au[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int a = arow[ty * TM + i];
+    if (a < 0) continue;
+    const float s = scale_input ? sel_w[a] : 1.f;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + tx * TN + j;
+      if (n < F) act[(size_t)a * F + n] = maybe_round(silu_f(s * ag[i][j]) * (s * au[i][j]), round);
+    }
+  }
+}
+
+// out[a, n] = (down_e act[a])[n] (times the assignment's weight unless scale_input)
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(
+    const float* __restrict__ act, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const T* __restrict__ Wd,
+    float* __restrict__ out, int N, int K, int scale_input) {
+  constexpr int BM = kMoeBM, BN = 64, BK = 16, TM = 2, TN = 4;
+  if ((int)blockIdx.y >= n_tiles[0]) return;
+  __shared__ float xs[BK][BM + 1];
+  __shared__ float ws[BK][BN + 1];
+  __shared__ int arow[BM];
+  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  const int tid = threadIdx.x, tx = tid % (BN / TN), ty = tid / (BN / TN);
+  const int n0 = blockIdx.x * BN;
+  const T* W = Wd + (size_t)e * N * K;
+  if (tid < BM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  __syncthreads();
+  float acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int idx = tid; idx < BM * BK; idx += 256) {
+      const int m = idx / BK, kk = idx % BK;
+      const int a = arow[m];
+      xs[kk][m] = (a >= 0 && k0 + kk < K) ? act[(size_t)a * K + k0 + kk] : 0.f;
+    }
+    for (int idx = tid; idx < BN * BK; idx += 256) {
+      const int n = idx / BK, kk = idx % BK;
+      ws[kk][n] = (n0 + n < N && k0 + kk < K) ? ld_f(W + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = xs[kk][ty * TM + i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = ws[kk][tx * TN + j];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int a = arow[ty * TM + i];
+    if (a < 0) continue;
+    const float s = scale_input ? 1.f : sel_w[a];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + tx * TN + j;
+      if (n < N) out[(size_t)a * N + n] = s * acc[i][j];
+    }
+  }
+}
+
+struct MoeScratch {
+  size_t cnt, n_tiles, perm, tiles, act, total;
+};
+inline size_t al256(size_t v) { return (v + 255) & ~(size_t)255; }
+MoeScratch moe_plan(int n_rows, int top, int E, int F) {
+  MoeScratch s;
+  const size_t n = (size_t)n_rows * top;
+  size_t off = 0;
+  s.cnt = off;     off += al256(sizeof(int32_t) * E);
+  s.n_tiles = off; off += al256(sizeof(int32_t));
+  s.perm = off;    off += al256(sizeof(int32_t) * n);
+  s.tiles = off;   off += al256(sizeof(int32_t) * 3 * (n / kMoeBM + E + 1));
+  s.act = off;     off += al256(sizeof(float) * n * F);
+  s.total = off;
+  return s;
+}
+
+// ------------------------------------------------------------------ residual update, norm on the output
+template <typename T>
+__global__ void postnorm_residual_kernel(float* __restrict__ x, const float* __restrict__ a, int n_a, float sa,
+                                         const float* __restrict__ b, float sb, const T* __restrict__ w, float eps,
+                                         bf16_t* __restrict__ x_b, int W) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  auto term = [&](int c) {
+    float v = a[((size_t)r * n_a) * W + c];
+    for (int j = 1; j < n_a; ++j) v += a[((size_t)r * n_a + j) * W + c];
+    v *= sa;
+    if (b) v += sb * b[(size_t)r * W + c];
+    return v;
+  };
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = term(c);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float xn = x[(size_t)r * W + c] + term(c) * rstd * ld_f(w + c);
+    x[(size_t)r * W + c] = xn;
+    if (x_b) x_b[(size_t)r * W + c] = (bf16_t)xn;
+  }
+}
+
+__global__ void scale_rows_kernel(float* __restrict__ x, int64_t ld, float s, int n_cols) {
+  const int r = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n_cols; c += gridDim.y * blockDim.x)
+    x[(size_t)r * ld + c] *= s;
+}
+
+}  // namespace
+
+// ====================================================================== C entry points
+extern "C" int sd_embed_hashed(const int32_t* tokens, const int32_t* prev_tokens, const void* table,
+                               const void* bigram, int w_f32, float scale, int buckets, int mul_prev, int mul_cur,
+                               float* x, void* x_bf16, int n_rows, int W, int vocab, sd_stream_t stream) {
+  SD_REQUIRE(tokens && table && x && n_rows >= 1 && W >= 1 && vocab >= 1, SD_ERR_INVALID, "sd_embed_hashed: bad argument");
+  SD_REQUIRE(!bigram || buckets >= 1, SD_ERR_INVALID, "sd_embed_hashed: a bigram table needs buckets >= 1");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32)
+    embed_hashed_kernel<float><<<n_rows, 256, 0, st>>>(tokens, prev_tokens, (const float*)table, (const float*)bigram,
+                                                       scale, buckets, mul_prev, mul_cur, x, (bf16_t*)x_bf16, W, vocab);
+  else
+    embed_hashed_kernel<bf16_t><<<n_rows, 256, 0, st>>>(tokens, prev_tokens, (const bf16_t*)table, (const bf16_t*)bigram,
+                                                        scale, buckets, mul_prev, mul_cur, x, (bf16_t*)x_bf16, W, vocab);
+  SD_CHECK_LAUNCH("sd_embed_hashed");
+  return SD_OK;
+}
+
+extern "C" int sd_rmsnorm_parts(const float* x, int64_t ldx, const float* gate, int64_t ldg, const void* w, int w_f32,
+                                float eps, float* out, int64_t ldo, void* out_bf16, int64_t ldob, int n_rows,
+                                int width, int parts, int round_bf16_out, sd_stream_t stream) {
+  SD_REQUIRE(x && out && n_rows >= 1 && width >= 1 && parts >= 1 && width % parts == 0 && ldx >= width && ldo >= width,
+             SD_ERR_INVALID, "sd_rmsnorm_parts: bad argument (width %d in %d parts)", width, parts);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, parts);
+  const int pw = width / parts;
+  if (w_f32)
+    rmsnorm_parts_kernel<float><<<grid, 256, 0, st>>>(x, ldx, gate, ldg, (const float*)w, eps, out, ldo,
+                                                      (bf16_t*)out_bf16, ldob, pw, round_bf16_out);
+  else
+    rmsnorm_parts_kernel<bf16_t><<<grid, 256, 0, st>>>(x, ldx, gate, ldg, (const bf16_t*)w, eps, out, ldo,
+                                                       (bf16_t*)out_bf16, ldob, pw, round_bf16_out);
+  SD_CHECK_LAUNCH("sd_rmsnorm_parts");
+  return SD_OK;
+}
+
+extern "C" int sd_rope_copy_rows(const float* src, int64_t ld_src, int src_head_stride, int src_offset, float* dst,
+                                 int64_t ld_dst, int dst_head_stride, int dst_offset, const int32_t* row_pos,
+                                 int n_rows, int heads, int n, int rot_dims, int rot_layout, const double* inv_freq,
+                                 float mag, sd_stream_t stream) {
+  SD_REQUIRE(src && dst && row_pos && n_rows >= 1 && heads >= 1 && src_offset >= 0 && dst_offset >= 0 && n >= 0,
+             SD_ERR_INVALID, "sd_rope_copy_rows: bad argument");
+  SD_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= n && (rot_dims == 0 || inv_freq), SD_ERR_INVALID,
+             "sd_rope_copy_rows: rot_dims %d must be even, at most %d, with a frequency table", rot_dims, n);
+  if (n == 0 || (rot_dims == 0 && src == dst)) return SD_OK;
+  rope_copy_kernel<<<dim3(n_rows, heads), 64, 0, (hipStream_t)stream>>>(src, ld_src, src_head_stride, src_offset, dst,
+                                                                        ld_dst, dst_head_stride, dst_offset, row_pos, n,
+                                                                        rot_dims, rot_layout, inv_freq, mag);
+  SD_CHECK_LAUNCH("sd_rope_copy_rows");
+  return SD_OK;
+}
+
+extern "C" int sd_rope_rows(float* x, int64_t ld, const int32_t* row_pos, int n_rows, int heads, int head_stride,
+                            int offset, int rot_dims, int rot_layout, const double* inv_freq, float mag,
+                            sd_stream_t stream) {
+  return sd_rope_copy_rows(x, ld, head_stride, offset, x, ld, head_stride, offset, row_pos, n_rows, heads, rot_dims,
+                           rot_dims, rot_layout, inv_freq, mag, stream);
+}
+
+extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, void* k_cache, void* v_cache,
+                               int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
+                               const int32_t* block_tables, int max_blocks, int page, int n_rows, int G, int dk, int dv,
+                               sd_stream_t stream) {
+  SD_REQUIRE(k && k_cache && row_pos && row_slot && block_tables && n_rows >= 1 && G >= 1 && dk >= 1 && page >= 1 &&
+                 max_blocks >= 1 && (!v || (v_cache && dv >= 1)),
+             SD_ERR_INVALID, "sd_cache_append: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, G);
+  if (cache_f32)
+    cache_append_kernel<float><<<grid, 128, 0, st>>>(k, ldk, v, ldv, (float*)k_cache, (float*)v_cache, row_pos, row_slot,
+                                                     block_tables, max_blocks, page, G, dk, dv);
+  else
+    cache_append_kernel<bf16_t><<<grid, 128, 0, st>>>(k, ldk, v, ldv, (bf16_t*)k_cache, (bf16_t*)v_cache, row_pos,
+                                                      row_slot, block_tables, max_blocks, page, G, dk, dv);
+  SD_CHECK_LAUNCH("sd_cache_append");
+  return SD_OK;
+}
+
+extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                           int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
+                                           const int32_t* block_tables, int max_blocks, int page, int n_rows, int H,
+                                           int G, int dk, int dv, int window, int keep_first, float scale, float* out,
+                                           void* out_bf16, sd_stream_t stream) {
+  SD_REQUIRE(q && k_cache && row_pos && row_slot && block_tables && out, SD_ERR_INVALID,
+             "sd_window_softmax_attention: null argument");
+  SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && keep_first >= 0 && page >= 1,
+             SD_ERR_INVALID, "sd_window_softmax_attention: bad shape");
+  SD_REQUIRE(dv >= 1 && dv <= 512 && (v_cache || dv <= dk), SD_ERR_UNSUPPORTED,
+             "sd_window_softmax_attention: value size %d outside 1..512 (or above the key row it is part of)", dv);
+  hipStream_t st = (hipStream_t)stream;
+  const int qh = H / G;
+  const int NH = qh <= 1 ? 1 : (qh <= 2 ? 2 : (qh <= 4 ? 4 : 8));
+  const int n_hgroups = (qh + NH - 1) / NH;
+  const int nc = dv <= 64 ? 1 : (dv <= 128 ? 2 : (dv <= 256 ? 4 : 8));
+  const size_t lds = sizeof(unsigned long long) * kTile +
+                     sizeof(float) * ((size_t)NH * kTile + (size_t)NH * dk + 3 * (size_t)NH + (size_t)4 * dv);
+  SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_softmax_attention: dim %d / vdim %d need %zu bytes of LDS",
+             dk, dv, lds);
+  const void* vc = v_cache ? v_cache : k_cache;
+  const int v_row = v_cache ? dv : dk;
+  dim3 grid(n_rows, G, n_hgroups);
+#define SD_NH(T, N)                                                                                              \
+  launch_softmax_nc<T, N>(grid, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables, max_blocks, \
+                          page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups)
+#define SD_T(T)                      \
+  do {                               \
+    if (NH == 1) SD_NH(T, 1);        \
+    else if (NH == 2) SD_NH(T, 2);   \
+    else if (NH == 4) SD_NH(T, 4);   \
+    else SD_NH(T, 8);                \
+  } while (0)
+  if (cache_f32) SD_T(float);
+  else SD_T(bf16_t);
+#undef SD_T
+#undef SD_NH
+  SD_CHECK_LAUNCH("sd_window_softmax_attention");
+  return SD_OK;
+}
+
+extern "C" int sd_causal_conv_rows(const float* x, int64_t ldx, const void* w, const void* b, int w_f32,
+                                   float* conv_state, const int32_t* row_pos, const int32_t* row_slot,
+                                   const int32_t* entries, int n_entries, float* out, int64_t ldo, int n_rows, int C,
+                                   int taps, int act, sd_stream_t stream) {
+  SD_REQUIRE(x && w && conv_state && row_pos && row_slot && entries && out && n_entries >= 1 && n_rows >= 1 && C >= 1 &&
+                 taps >= 1 && ldx >= C && ldo >= C,
+             SD_ERR_INVALID, "sd_causal_conv_rows: bad argument");
+  SD_REQUIRE(out != x, SD_ERR_INVALID, "sd_causal_conv_rows: not in place (rows read their predecessors)");
+  hipStream_t st = (hipStream_t)stream;
+  const int cb = (C + 255) / 256;
+  if (w_f32)
+    causal_conv_rows_kernel<float><<<dim3(n_rows, cb), 256, 0, st>>>(x, ldx, (const float*)w, (const float*)b, conv_state,
+                                                                     row_pos, row_slot, out, ldo, C, taps, act);
+  else
+    causal_conv_rows_kernel<bf16_t><<<dim3(n_rows, cb), 256, 0, st>>>(x, ldx, (const bf16_t*)w, (const bf16_t*)b,
+                                                                      conv_state, row_pos, row_slot, out, ldo, C, taps, act);
+  SD_CHECK_LAUNCH("sd_causal_conv_rows");
+  if (taps > 1) {
+    conv_state_update_kernel<<<dim3(n_entries, cb), 256, 0, st>>>(x, ldx, conv_state, entries, C, taps);
+    SD_CHECK_LAUNCH("sd_causal_conv_rows (state)");
+  }
+  return SD_OK;
+}
+
+extern "C" int sd_ssd_steps(const float* dt, int64_t ld, const void* dt_bias, const void* a_log, int w_f32, float* step,
+                            float* decay, int n_rows, int H, sd_stream_t stream) {
+  SD_REQUIRE(dt && dt_bias && a_log && step && decay && n_rows >= 1 && H >= 1 && ld >= H, SD_ERR_INVALID,
+             "sd_ssd_steps: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  const int n = n_rows * H;
+  if (w_f32)
+    ssd_steps_kernel<float><<<(n + 255) / 256, 256, 0, st>>>(dt, ld, (const float*)dt_bias, (const float*)a_log, step, decay, n, H);
+  else
+    ssd_steps_kernel<bf16_t><<<(n + 255) / 256, 256, 0, st>>>(dt, ld, (const bf16_t*)dt_bias, (const bf16_t*)a_log, step, decay, n, H);
+  SD_CHECK_LAUNCH("sd_ssd_steps");
+  return SD_OK;
+}
+
+extern "C" int sd_decay_scan_rows(const float* q, const float* k, int64_t ldqk, const float* v, int64_t ldv,
+                                  const float* decay, const float* k_scale, const void* skip, int w_f32, float* state,
+                                  const int32_t* entries, int n_entries, float* out, int H, int Gq, int dk, int dv,
+                                  sd_stream_t stream) {
+  SD_REQUIRE(q && k && v && decay && state && entries && out && n_entries >= 1 && H >= 1 && Gq >= 1 && H % Gq == 0 &&
+                 dv >= 1,
+             SD_ERR_INVALID, "sd_decay_scan_rows: bad argument");
+  SD_REQUIRE(dk >= 1 && dk <= 256, SD_ERR_UNSUPPORTED, "sd_decay_scan_rows: key size %d outside 1..256", dk);
+  SD_REQUIRE(H <= 4096, SD_ERR_UNSUPPORTED, "sd_decay_scan_rows: more than 4096 heads");
+  const int NS = (dk + kStrip - 1) / kStrip;
+  hipStream_t st = (hipStream_t)stream;
+  int CT = 256 / NS;
+  if (CT > dv) CT = dv;
+  if (CT > 64) CT = 64;
+  const int tiles = (dv + CT - 1) / CT;
+  const int dkp = NS * kStrip;
+  int CH = kScanLoads * (CT * NS) / dkp;
+  if (CH > kScanChunk) CH = kScanChunk;
+  SD_REQUIRE(CH >= 1 && CH * CT <= kScanLoadsV * CT * NS, SD_ERR_UNSUPPORTED,
+             "sd_decay_scan_rows: key size %d with value size %d leaves no chunk", dk, dv);
+  const size_t lds = sizeof(float) * ((size_t)2 * CH * dkp + (size_t)CH * CT + 2 * (size_t)CH + (size_t)CH * NS * CT);
+  dim3 grid(tiles, H, n_entries);
+  const int hpg = H / Gq;
+  if (w_f32)
+    decay_scan_rows_kernel<float><<<grid, CT * NS, lds, st>>>(q, k, ldqk, v, ldv, decay, k_scale, (const float*)skip,
+                                                              state, entries, out, H, hpg, dk, dv, CT, NS, CH);
+  else
+    decay_scan_rows_kernel<bf16_t><<<grid, CT * NS, lds, st>>>(q, k, ldqk, v, ldv, decay, k_scale, (const bf16_t*)skip,
+                                                               state, entries, out, H, hpg, dk, dv, CT, NS, CH);
+  SD_CHECK_LAUNCH("sd_decay_scan_rows");
+  return SD_OK;
+}
+
+extern "C" int sd_moe_route(const float* logits, int64_t ld, int32_t* sel_expert, float* sel_weight, int n_rows, int E,
+                            int top, int score_kind, int renorm, sd_stream_t stream) {
+  SD_REQUIRE(logits && sel_expert && sel_weight && n_rows >= 1 && E >= 1 && top >= 1 && top <= E && ld >= E,
+             SD_ERR_INVALID, "sd_moe_route: bad argument (E=%d top=%d)", E, top);
+  SD_REQUIRE(E <= 8192, SD_ERR_UNSUPPORTED, "sd_moe_route: more than 8192 experts");
+  moe_route_kernel<<<n_rows, 64, sizeof(float) * E, (hipStream_t)stream>>>(logits, ld, sel_expert, sel_weight, E, top,
+                                                                           score_kind, renorm);
+  SD_CHECK_LAUNCH("sd_moe_route");
+  return SD_OK;
+}
+
+extern "C" size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W) {
+  (void)W;
+  if (n_rows < 1 || top < 1 || E < 1 || F < 1) return 0;
+  return moe_plan(n_rows, top, E, F).total;
+}
+
+extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_expert, const float* sel_weight,
+                              const void* w_gate_up, const void* w_down, int w_f32, float* out, int n_rows, int top,
+                              int E, int F, int W, int scale_input, int act_kind, void* scratch, size_t scratch_bytes,
+                              sd_stream_t stream) {
+  SD_REQUIRE(x && sel_expert && sel_weight && w_gate_up && w_down && out && scratch, SD_ERR_INVALID,
+             "sd_moe_experts: null argument");
+  SD_REQUIRE(n_rows >= 1 && top >= 1 && E >= 1 && F >= 1 && W >= 1 && ldx >= W, SD_ERR_INVALID, "sd_moe_experts: bad shape");
+  SD_REQUIRE(act_kind == 0, SD_ERR_UNSUPPORTED, "sd_moe_experts: activation %d is not provided", act_kind);
+  const MoeScratch p = moe_plan(n_rows, top, E, F);
+  SD_REQUIRE(scratch_bytes >= p.total, SD_ERR_WORKSPACE, "sd_moe_experts: scratch %zu < %zu bytes", scratch_bytes, p.total);
+  SD_REQUIRE(sd_aligned16(scratch), SD_ERR_INVALID, "sd_moe_experts: scratch unaligned");
+  hipStream_t st = (hipStream_t)stream;
+  char* base = (char*)scratch;
+  int32_t* cnt = (int32_t*)(base + p.cnt);
+  int32_t* n_tiles = (int32_t*)(base + p.n_tiles);
+  int32_t* perm = (int32_t*)(base + p.perm);
+  int32_t* tiles = (int32_t*)(base + p.tiles);
+  float* act = (float*)(base + p.act);
+  const int n = n_rows * top;
+  moe_count_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt);
+  SD_CHECK_LAUNCH("sd_moe_experts (count)");
+  moe_group_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt, E, perm, tiles, n_tiles);
+  SD_CHECK_LAUNCH("sd_moe_experts (group)");
+  const int max_tiles = n / kMoeBM + E;
+  const int tiles_y = max_tiles < (n + 0) ? max_tiles : n;   // never more tiles than assignments
+  if (w_f32) {
+    moe_gate_up_kernel<float><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
+                                                                            (const float*)w_gate_up, act, top, F, W, scale_input, 0);
+    SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
+    moe_down_kernel<float><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
+                                                                         (const float*)w_down, out, W, F, scale_input);
+  } else {
+    moe_gate_up_kernel<bf16_t><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
+                                                                             (const bf16_t*)w_gate_up, act, top, F, W, scale_input, 1);
+    SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
+    moe_down_kernel<bf16_t><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
+                                                                          (const bf16_t*)w_down, out, W, F, scale_input);
+  }
+  SD_CHECK_LAUNCH("sd_moe_experts (down)");
+  return SD_OK;
+}
+
+extern "C" int sd_postnorm_residual(float* x, const float* a, int n_a, float sa, const float* b, float sb, const void* w,
+                                    int w_f32, float eps, void* x_bf16, int n_rows, int W, sd_stream_t stream) {
+  SD_REQUIRE(x && a && w && n_a >= 1 && n_rows >= 1 && W >= 1, SD_ERR_INVALID, "sd_postnorm_residual: bad argument");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32)
+    postnorm_residual_kernel<float><<<n_rows, 256, 0, st>>>(x, a, n_a, sa, b, sb, (const float*)w, eps, (bf16_t*)x_bf16, W);
+  else
+    postnorm_residual_kernel<bf16_t><<<n_rows, 256, 0, st>>>(x, a, n_a, sa, b, sb, (const bf16_t*)w, eps, (bf16_t*)x_bf16, W);
+  SD_CHECK_LAUNCH("sd_postnorm_residual");
+  return SD_OK;
+}
+
+extern "C" int sd_scale_rows(float* x, int64_t ld, float s, int n_rows, int n_cols, sd_stream_t stream) {
+  SD_REQUIRE(x && n_rows >= 1 && n_cols >= 1 && ld >= n_cols, SD_ERR_INVALID, "sd_scale_rows: bad argument");
+  int by = (n_cols + 255) / 256;
+  if (by > 64) by = 64;
+  scale_rows_kernel<<<dim3(n_rows, by), 256, 0, (hipStream_t)stream>>>(x, ld, s, n_cols);
+  SD_CHECK_LAUNCH("sd_scale_rows");
+  return SD_OK;
+}

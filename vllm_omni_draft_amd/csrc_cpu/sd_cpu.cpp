@@ -1492,6 +1492,46 @@ extern "C" int sd_gated_residual_norm(float*, const float*, const float*, int64_
 extern "C" int sd_relu_mul_rows(const float*, const float*, int64_t, void*, int, int, sd_stream_t) {
   UNSUPPORTED("sd_relu_mul_rows");
 }
+extern "C" int sd_matmul_rows_batched(const float*, int64_t, int64_t, const void*, int, int64_t, float*, int64_t,
+                                      int64_t, void*, int, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_matmul_rows_batched");
+}
+extern "C" int sd_embed_hashed(const int32_t*, const int32_t*, const void*, const void*, int, float, int, int, int,
+                               float*, void*, int, int, int, sd_stream_t) { UNSUPPORTED("sd_embed_hashed"); }
+extern "C" int sd_rmsnorm_parts(const float*, int64_t, const float*, int64_t, const void*, int, float, float*, int64_t,
+                                void*, int64_t, int, int, int, int, sd_stream_t) { UNSUPPORTED("sd_rmsnorm_parts"); }
+extern "C" int sd_rope_rows(float*, int64_t, const int32_t*, int, int, int, int, int, int, const double*, float,
+                            sd_stream_t) { UNSUPPORTED("sd_rope_rows"); }
+extern "C" int sd_rope_copy_rows(const float*, int64_t, int, int, float*, int64_t, int, int, const int32_t*, int, int,
+                                 int, int, int, const double*, float, sd_stream_t) { UNSUPPORTED("sd_rope_copy_rows"); }
+extern "C" int sd_cache_append(const float*, int64_t, const float*, int64_t, void*, void*, int, const int32_t*,
+                               const int32_t*, const int32_t*, int, int, int, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_cache_append");
+}
+extern "C" int sd_window_softmax_attention(const float*, int64_t, const void*, const void*, int, const int32_t*,
+                                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int,
+                                           float, float*, void*, sd_stream_t) {
+  UNSUPPORTED("sd_window_softmax_attention");
+}
+extern "C" int sd_causal_conv_rows(const float*, int64_t, const void*, const void*, int, float*, const int32_t*,
+                                   const int32_t*, const int32_t*, int, float*, int64_t, int, int, int, int,
+                                   sd_stream_t) { UNSUPPORTED("sd_causal_conv_rows"); }
+extern "C" int sd_ssd_steps(const float*, int64_t, const void*, const void*, int, float*, float*, int, int,
+                            sd_stream_t) { UNSUPPORTED("sd_ssd_steps"); }
+extern "C" int sd_decay_scan_rows(const float*, const float*, int64_t, const float*, int64_t, const float*,
+                                  const float*, const void*, int, float*, const int32_t*, int, float*, int, int, int,
+                                  int, sd_stream_t) { UNSUPPORTED("sd_decay_scan_rows"); }
+extern "C" int sd_moe_route(const float*, int64_t, int32_t*, float*, int, int, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_moe_route");
+}
+extern "C" size_t sd_moe_experts_scratch_bytes(int, int, int, int, int) { return 0; }
+extern "C" int sd_moe_experts(const float*, int64_t, const int32_t*, const float*, const void*, const void*, int,
+                              float*, int, int, int, int, int, int, int, void*, size_t, sd_stream_t) {
+  UNSUPPORTED("sd_moe_experts");
+}
+extern "C" int sd_postnorm_residual(float*, const float*, int, float, const float*, float, const void*, int, float,
+                                    void*, int, int, sd_stream_t) { UNSUPPORTED("sd_postnorm_residual"); }
+extern "C" int sd_scale_rows(float*, int64_t, float, int, int, sd_stream_t) { UNSUPPORTED("sd_scale_rows"); }
 extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc*) {
   set_error("sd_seq_model_create: not provided by the CPU build of the library");
   return nullptr;

@@ -146,7 +146,9 @@ class SeqCache:
     when the slot is taken again (a sequence that starts at position 0 starts from zero).
     Window layers: k / v [pages, kv_heads, PAGE, dim | vdim] in the serving dtype and the pooled
     means pk / pv f32 [pages, kv_heads, pooled slots per page, dim | vdim]; one page table per
-    slot serves all window layers."""
+    slot serves all window layers.  Latent attention keeps one row [kv_rank + rot_dim] per token
+    in k only; a state-space recurrence keeps state[layer] [slots, heads, state, vdim] and the
+    tail of its convolution's inputs conv[layer] f32 [slots, taps - 1, channels]."""
 
     def __init__(self, cfg, dtype: torch.dtype, max_seqs: int, num_pages: int, max_seq_len: int,
                  device="cuda"):
@@ -163,10 +165,23 @@ class SeqCache:
         self.v: Dict[int, torch.Tensor] = {}
         self.pk: Dict[int, torch.Tensor] = {}
         self.pv: Dict[int, torch.Tensor] = {}
+        self.conv: Dict[int, torch.Tensor] = {}
         self.has_pages = False
         for i, l in enumerate(cfg.layers):
             m = l.mixer
-            if m.kind == "attention":
+            if m.kind == "latent_attention":
+                # one row per token serves as key and value: the latent, then the shared rotated part
+                self.has_pages = True
+                self.k[i] = torch.zeros(num_pages, 1, PAGE, m.kv_rank + m.rot_dim, dtype=dtype, device=device)
+            elif m.kind == "parallel":
+                self.has_pages = True
+                sd = m.ssd
+                self.k[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.dim, dtype=dtype, device=device)
+                self.v[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.vdim, dtype=dtype, device=device)
+                self.state[i] = torch.zeros(max_seqs, sd.heads, sd.state, sd.vdim, dtype=torch.float32, device=device)
+                self.conv[i] = torch.zeros(max_seqs, max(sd.taps - 1, 1), sd.conv_channels, dtype=torch.float32,
+                                           device=device)
+            elif m.kind == "attention":
                 self.has_pages = True
                 ps = ops.pooled_slots_per_page(PAGE, m.pool)
                 self.k[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.dim, dtype=dtype, device=device)
@@ -203,5 +218,5 @@ class SeqCache:
         self.slots.free(slot)
 
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for d in (self.state, self.k, self.v, self.pk, self.pv)
+        return sum(t.numel() * t.element_size() for d in (self.state, self.k, self.v, self.pk, self.pv, self.conv)
                    for t in d.values())

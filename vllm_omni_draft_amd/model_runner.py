@@ -201,7 +201,7 @@ class DecoderModel:
 
 
 # ---------------------------------------------------------------------------------------------
-_MIX_KIND = {"retention": 0, "gla": 1, "attention": 2}
+_MIX_KIND = {"retention": 0, "gla": 1, "attention": 2, "latent_attention": 3, "parallel": 4}
 
 
 class SeqModel:
@@ -229,6 +229,27 @@ class SeqModel:
 
         for i, (spec, t) in enumerate(zip(cfg.layers, weights.layers)):
             m = spec.mixer
+            if cfg.block == "postnorm":
+                sd, ex = m.ssd, spec.experts
+                layers[i] = _lib.SeqLayer(
+                    kind=_MIX_KIND[m.kind], block=1, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
+                    rot_dims=m.rot_dims, rot_layout=1, inv_freq=_ptr(t.inv_freq), rot_mag=t.rot_mag,
+                    score_scale=m.scale, window=m.window, keep_first=m.keep_first,
+                    norm_w=_ptr(t.norm_w), norm2_w=_ptr(t.norm2_w), w_in=rm(t.w_in), w_in_tiled=tl(t.w_in),
+                    w_o=rm(t.w_o), w_o_tiled=tl(t.w_o),
+                    q_rank=m.q_rank, kv_rank=m.kv_rank, rot_dim=m.rot_dim, dq_norm_w=_ptr(t.dq_norm_w),
+                    dkv_norm_w=_ptr(t.dkv_norm_w), w_uq=rm(t.w_uq), w_uq_tiled=tl(t.w_uq), w_uk_t=_ptr(t.w_uk_t),
+                    w_uv=_ptr(t.w_uv), q_norm_w=_ptr(t.q_norm_w), k_norm_w=_ptr(t.k_norm_w),
+                    left_scale=m.left_scale, right_scale=m.right_scale,
+                    s_heads=sd.heads if sd else 0, s_vdim=sd.vdim if sd else 0, s_state=sd.state if sd else 0,
+                    s_groups=sd.groups if sd else 0, s_taps=sd.taps if sd else 0,
+                    s_norm_groups=sd.norm_groups if sd else 0, conv_w=_ptr(t.conv_w), conv_b=_ptr(t.conv_b),
+                    dt_bias=_ptr(t.dt_bias), a_log=_ptr(t.a_log), skip_d=_ptr(t.skip_d), s_norm_w=_ptr(t.s_norm_w),
+                    w_o2=rm(t.w_o2), w_o2_tiled=tl(t.w_o2), state=_ptr(cache.state.get(i)),
+                    conv_state=_ptr(cache.conv.get(i)), k_cache=_ptr(cache.k.get(i)), v_cache=_ptr(cache.v.get(i)),
+                    n_experts=ex.experts if ex else 0, top=ex.top if ex else 0, expert_ff=ex.ff if ex else 0,
+                    w_router=_ptr(t.w_router), w_gate_up=_ptr(t.w_gate_up), w_down_e=_ptr(t.w_down_e))
+                continue
             rec = m.kind != "attention"
             layers[i] = _lib.SeqLayer(
                 kind=_MIX_KIND[m.kind], heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
@@ -247,7 +268,12 @@ class SeqModel:
                 pk_cache=_ptr(cache.pk.get(i)), pv_cache=_ptr(cache.pv.get(i)))
         desc = _lib.SeqModelDesc(n_layers=cfg.n_layers, width=cfg.width, vocab=cfg.vocab,
                                  weights_f32=int(f32), norm_eps=cfg.norm_eps, embed=_ptr(weights.embed),
-                                 head_tiled=tl(weights.head_tiled), final_norm_w=_ptr(weights.final_norm_w), layers=layers)
+                                 head_tiled=tl(weights.head_tiled), final_norm_w=_ptr(weights.final_norm_w), layers=layers,
+                                 plain_norm=int(cfg.block == "postnorm"), embed_scale=cfg.embed_scale,
+                                 bigram=_ptr(weights.bigram), buckets=(cfg.bigram or {}).get("buckets", 0),
+                                 mul_prev=(cfg.bigram or {}).get("mul_prev", 0),
+                                 mul_cur=(cfg.bigram or {}).get("mul_cur", 0), head=_ptr(weights.head),
+                                 logit_scale=cfg.logit_scale)
         self._handle = _lib.load().sd_seq_model_create(C.byref(desc))
         if not self._handle:
             raise _lib.SdError(f"sd_seq_model_create failed: {_lib.last_error()}")
@@ -272,10 +298,16 @@ class SeqModel:
         self.workspace = torch.empty(int(n), dtype=torch.uint8, device=self.weights.embed.device)
 
     def forward(self, n_rows: int, n_entries: int, tokens, row_pos, row_slot, entries, n_out: int,
-                out_rows, logits, layer_out=None) -> None:
+                out_rows, logits, layer_out=None, prev_tokens=None) -> None:
         """int32 device tensors tokens / row_pos / row_slot [n_rows], entries [n_entries, 4]
         {slot, first row, rows, first position}, out_rows [n_out]; logits f32 [n_out, vocab];
-        layer_out (optional) f32 [n_layers, n_rows, width] receives the residual after each layer."""
+        layer_out (optional) f32 [n_layers, n_rows, width] receives the residual after each layer;
+        prev_tokens int32 [n_rows] (models with a bigram table): the token before each row in its
+        sequence, -1 for a sequence's first."""
+        if self.cfg.bigram is not None:
+            if prev_tokens is None or prev_tokens.dtype != torch.int32 or not prev_tokens.is_contiguous() \
+                    or not prev_tokens.is_cuda or prev_tokens.numel() < n_rows:
+                raise _lib.SdError("this model needs prev_tokens: a contiguous int32 device tensor [n_rows]")
         for t, name in ((tokens, "tokens"), (row_pos, "row_pos"), (row_slot, "row_slot"), (entries, "entries")):
             if t.dtype != torch.int32 or not t.is_contiguous() or not t.is_cuda:
                 raise _lib.SdError(f"{name} must be a contiguous int32 device tensor")
@@ -296,7 +328,8 @@ class SeqModel:
                               entries=entries.data_ptr(), block_tables=c.block_tables.data_ptr(),
                               max_blocks=c.max_blocks_per_seq, page=c.page, n_out=n_out,
                               out_rows=_ptr(out_rows) if n_out else None,
-                              logits=_ptr(logits) if n_out else None, layer_out=_ptr(layer_out))
+                              logits=_ptr(logits) if n_out else None, layer_out=_ptr(layer_out),
+                              prev_tokens=_ptr(prev_tokens))
         rc = _lib.load().sd_seq_model_forward(self._handle, C.byref(batch), self.workspace.data_ptr(),
                                               self.workspace.numel(), ops._stream())
         _lib.check(rc, "sd_seq_model_forward")

@@ -44,6 +44,7 @@ class SeqEngineConfig:
 class _Seq:
     slot: int
     n: int = 0                   # tokens computed so far
+    last: int = -1               # the last token computed (-1: none yet): part of the sequence's state
 
 
 class SeqEngine:
@@ -133,6 +134,7 @@ class SeqEngine:
         self.stream.synchronize()
         for s, t, _ in plan:
             s.n += len(t)
+            s.last = int(t[-1])
         return (logits, trace) if layer_out else logits
 
     def _run_passes(self, plan, done, out_at, logits, trace) -> None:
@@ -141,6 +143,7 @@ class SeqEngine:
             toks: List[int] = []
             pos: List[int] = []
             slot: List[int] = []
+            prev: List[int] = []
             ents: List[int] = []
             out_rows: List[int] = []
             out_dst: List[int] = []
@@ -154,13 +157,14 @@ class SeqEngine:
                 toks += t[lo:hi]
                 pos += range(s.n + lo, s.n + hi)
                 slot += [s.slot] * (hi - lo)
+                prev += [t[lo - 1] if lo > 0 else s.last] + t[lo:hi - 1]
                 for j, wi in enumerate(w):
                     if lo <= wi < hi:
                         out_rows.append(row0 + wi - lo)
                         out_dst.append(out_at[i] + j)
                 room -= hi - lo
                 done[i] = hi
-            self._run_pass(toks, pos, slot, ents, out_rows, out_dst, logits, trace)
+            self._run_pass(toks, pos, slot, prev, ents, out_rows, out_dst, logits, trace)
 
     def _drop_graphs(self) -> None:
         lib = _lib.load()
@@ -195,8 +199,9 @@ class SeqEngine:
             stream = ops._stream()
             _lib.check(lib.sd_graph_begin(stream), "sd_graph_begin")
             try:
-                self.model.forward(R, E, dev[0:R], dev[R:2 * R], dev[2 * R:3 * R], dev[3 * R:3 * R + 4 * E], O,
-                                   dev[3 * R + 4 * E:] if O else None, g["logits"] if O else None, None)
+                self.model.forward(R, E, dev[0:R], dev[R:2 * R], dev[2 * R:3 * R], dev[4 * R:4 * R + 4 * E], O,
+                                   dev[4 * R + 4 * E:] if O else None, g["logits"] if O else None, None,
+                                   dev[3 * R:4 * R])
             finally:
                 rc = lib.sd_graph_end(stream, C.byref(handle))
             _lib.check(rc, "sd_graph_end")
@@ -211,9 +216,9 @@ class SeqEngine:
         self.passes += 1
         return True
 
-    def _run_pass(self, toks, pos, slot, ents, out_rows, out_dst, logits, trace) -> None:
+    def _run_pass(self, toks, pos, slot, prev, ents, out_rows, out_dst, logits, trace) -> None:
         R, E, O = len(toks), len(ents) // 4, len(out_rows)
-        host = torch.tensor(toks + pos + slot + ents + out_rows, dtype=torch.int32)
+        host = torch.tensor(toks + pos + slot + prev + ents + out_rows, dtype=torch.int32)
         if self.cfg.use_graph and trace is None and R == E and R <= self.cfg.graph_max_rows:
             if self._run_graph_pass(host, R, E, O, out_dst, logits):
                 return
@@ -221,8 +226,9 @@ class SeqEngine:
         a = dev[0:R]
         b = dev[R:2 * R]
         c = dev[2 * R:3 * R]
-        e = dev[3 * R:3 * R + 4 * E]
-        o = dev[3 * R + 4 * E:]
+        p = dev[3 * R:4 * R]
+        e = dev[4 * R:4 * R + 4 * E]
+        o = dev[4 * R + 4 * E:]
         contiguous_out = O > 0 and out_dst == list(range(out_dst[0], out_dst[0] + O))
         V = self.model_cfg.vocab
         if O == 0:
@@ -231,7 +237,7 @@ class SeqEngine:
             dst = logits[out_dst[0]:out_dst[0] + O]
         else:
             dst = torch.empty(O, V, dtype=torch.float32, device=self.device)
-        self.model.forward(R, E, a, b, c, e, O, o if O else None, dst, trace)
+        self.model.forward(R, E, a, b, c, e, O, o if O else None, dst, trace, p)
         if O and not contiguous_out:
             logits[torch.tensor(out_dst, device=self.device)] = dst
         self.passes += 1

@@ -334,6 +334,26 @@ class SeqLayerTensors:
     head_bias: Optional[torch.Tensor] = None   # f32 [heads]
     head_norm_w: Optional[torch.Tensor] = None
     inv_freq: Optional[torch.Tensor] = None    # f64 [rot_dims / 2]
+    rot_mag: float = 1.0                       # factor of cos and sin
+    # layers normed on their sublayers' outputs (norm_w is norm1; r1_bias unused)
+    norm2_w: Optional[torch.Tensor] = None
+    dq_norm_w: Optional[torch.Tensor] = None   # latent attention
+    dkv_norm_w: Optional[torch.Tensor] = None
+    w_uq: object = None
+    w_uk_t: Optional[torch.Tensor] = None      # [heads, kv_rank, dim]: key expansions, transposed
+    w_uv: Optional[torch.Tensor] = None
+    q_norm_w: Optional[torch.Tensor] = None    # attention beside a state-space recurrence
+    k_norm_w: Optional[torch.Tensor] = None
+    conv_w: Optional[torch.Tensor] = None
+    conv_b: Optional[torch.Tensor] = None
+    dt_bias: Optional[torch.Tensor] = None
+    a_log: Optional[torch.Tensor] = None
+    skip_d: Optional[torch.Tensor] = None
+    s_norm_w: Optional[torch.Tensor] = None
+    w_o2: object = None
+    w_router: Optional[torch.Tensor] = None    # routed experts
+    w_gate_up: Optional[torch.Tensor] = None   # [experts, 2*ff, width]
+    w_down_e: Optional[torch.Tensor] = None    # [experts, width, ff]
 
 
 @dataclass
@@ -343,18 +363,23 @@ class SeqModelWeights:
     embed: torch.Tensor
     final_norm_w: torch.Tensor
     layers: List[SeqLayerTensors]
-    head_tiled: Optional["ops.TiledWeight"] = None   # the embedding table once more, tiled, as the head
+    head_tiled: Optional["ops.TiledWeight"] = None   # the head's matrix once more, tiled
+    head: Optional[torch.Tensor] = None              # an untied head, row-major
+    bigram: Optional[torch.Tensor] = None            # [buckets + 1, width]
 
     def tensors(self):
         yield self.embed
         yield self.final_norm_w
         if self.head_tiled is not None:
             yield self.head_tiled.data
+        for t in (self.head, self.bigram):
+            if t is not None:
+                yield t
         for l in self.layers:
             for t in vars(l).values():
                 if isinstance(t, ops.TiledWeight):
                     yield t.data
-                elif t is not None:
+                elif isinstance(t, torch.Tensor):
                     yield t
 
     def nbytes(self) -> int:
@@ -387,6 +412,16 @@ def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
         if tiled and dtype == torch.bfloat16 and t.shape[1] % 32 == 0 and torch.device(device).type == "cuda":
             return ops.tile_weights(d, ops.TILE_PLAIN)
         return d
+
+    if cfg.block == "postnorm":
+        layers = [_postnorm_layer(cfg, i, get, dev, mat) for i in range(cfg.n_layers)]
+        head_t = get("embed" if cfg.tied_head else "head", (cfg.vocab, W))
+        head = mat(head_t)
+        bg = cfg.bigram
+        return SeqModelWeights(cfg, dtype, dev(get("embed", (cfg.vocab, W))), dev(get("final.norm", (W,))), layers,
+                               head if isinstance(head, ops.TiledWeight) else None,
+                               None if cfg.tied_head else dev(head_t),
+                               dev(get("bigram", (bg["buckets"] + 1, W))) if bg else None)
 
     layers = []
     for i, l in enumerate(cfg.layers):
@@ -423,6 +458,49 @@ def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
                            head if isinstance(head, ops.TiledWeight) else None)
 
 
+def _postnorm_layer(cfg, i: int, get, dev, mat) -> SeqLayerTensors:
+    """Layer i of a model whose layers are normed on their sublayers' outputs: the matrices that
+    read the residual stacked into w_in, per-head key expansions transposed for the product
+    that takes a query to the latent, the experts' matrices stacked per layer."""
+    from .config import rotary_frequencies
+    l, p, W = cfg.layers[i], f"l{i}.", cfg.width
+    m = l.mixer
+    H, dk, dv = m.heads, m.dim, m.vdim
+    if m.kind == "latent_attention":
+        rk, dr, qr = m.kv_rank, m.rot_dim, m.q_rank
+        w_in = torch.cat([get(p + "mix.dq", (qr, W)).float(), get(p + "mix.dkv", (rk + dr, W)).float()])
+        lt = SeqLayerTensors(norm_w=dev(get(p + "norm1", (W,))), w_in=mat(w_in), w_o=mat(get(p + "mix.o", (W, H * dv))),
+                             r1_bias=None)
+        lt.dq_norm_w, lt.dkv_norm_w = dev(get(p + "mix.dq.norm", (qr,))), dev(get(p + "mix.dkv.norm", (rk,)))
+        lt.w_uq = mat(get(p + "mix.uq", (H * (dk + dr), qr)))
+        lt.w_uk_t = dev(get(p + "mix.uk", (H * dk, rk)).view(H, dk, rk).transpose(1, 2))
+        lt.w_uv = dev(get(p + "mix.uv", (H * dv, rk)))
+        if m.rot_dims:
+            f, mag = rotary_frequencies(m.rot_dims, m.rot_base, m.rot_scaling)
+            lt.inv_freq, lt.rot_mag = dev(f, torch.float64), float(mag)
+    else:
+        G, sd = m.kv_heads, m.ssd
+        w_in = torch.cat([get(p + "mix.left.q", (H * dk, W)).float(), get(p + "mix.left.k", (G * dk, W)).float(),
+                          get(p + "mix.left.v", (G * dv, W)).float(),
+                          get(p + "mix.right.in", (2 * sd.inner + 2 * sd.groups * sd.state + sd.heads, W)).float()])
+        lt = SeqLayerTensors(norm_w=dev(get(p + "norm1", (W,))), w_in=mat(w_in),
+                             w_o=mat(get(p + "mix.left.o", (W, H * dv))), r1_bias=None)
+        lt.q_norm_w, lt.k_norm_w = dev(get(p + "mix.left.q.norm", (H * dk,))), dev(get(p + "mix.left.k.norm", (G * dk,)))
+        lt.conv_w = dev(get(p + "mix.right.conv", (sd.conv_channels, sd.taps)))
+        lt.conv_b = dev(get(p + "mix.right.conv.b", (sd.conv_channels,)))
+        lt.dt_bias, lt.a_log = dev(get(p + "mix.right.dt_bias", (sd.heads,))), dev(get(p + "mix.right.A_log", (sd.heads,)))
+        lt.skip_d, lt.s_norm_w = dev(get(p + "mix.right.D", (sd.heads,))), dev(get(p + "mix.right.norm", (sd.inner,)))
+        lt.w_o2 = mat(get(p + "mix.right.o", (W, sd.inner)))
+    ex = l.experts
+    if ex is not None:
+        lt.norm2_w = dev(get(p + "norm2", (W,)))
+        lt.w_router = dev(get(p + "mlp.router", (ex.experts, W)))
+        lt.w_gate_up = dev(torch.stack([torch.cat([get(p + f"mlp.e{e}.gate", (ex.ff, W)), get(p + f"mlp.e{e}.up", (ex.ff, W))])
+                                        for e in range(ex.experts)]))
+        lt.w_down_e = dev(torch.stack([get(p + f"mlp.e{e}.down", (W, ex.ff)) for e in range(ex.experts)]))
+    return lt
+
+
 def seq_from_safetensors_dir(cfg, model_dir: str, device="cuda",
                              dtype: torch.dtype = torch.bfloat16) -> SeqModelWeights:
     from safetensors import safe_open
@@ -447,6 +525,8 @@ def seq_random_state(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
     def rn(*shape, s):
         return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
 
+    if cfg.block == "postnorm":
+        return _postnorm_random_state(cfg, rn)
     st = {"embed": rn(cfg.vocab, W, s=1.0), "final.norm": rn(W, s=0.1)}
     for i, l in enumerate(cfg.layers):
         m, p = l.mixer, f"l{i}."
@@ -467,6 +547,44 @@ def seq_random_state(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
             st[p + "mlp.gate"], st[p + "mlp.up"] = rn(l.ff, W, s=W ** -0.5), rn(l.ff, W, s=W ** -0.5)
             st[p + "mlp.down"] = rn(W, l.ff, s=l.ff ** -0.5)
             st[p + "rg2"], st[p + "rg2.b"] = rn(W, W, s=W ** -0.5), rn(W, s=0.5)
+    return st
+
+
+def _postnorm_random_state(cfg, rn) -> Dict[str, torch.Tensor]:
+    W = cfg.width
+    st = {"embed": rn(cfg.vocab, W, s=1.0), "final.norm": 1 + rn(W, s=0.1)}
+    if not cfg.tied_head:
+        st["head"] = rn(cfg.vocab, W, s=W ** -0.5)
+    if cfg.bigram:
+        st["bigram"] = rn(cfg.bigram["buckets"] + 1, W, s=0.5)
+    for i, l in enumerate(cfg.layers):
+        m, p = l.mixer, f"l{i}."
+        H, dk, dv = m.heads, m.dim, m.vdim
+        st[p + "norm1"] = 1 + rn(W, s=0.1)
+        if m.kind == "latent_attention":
+            rk, dr, qr = m.kv_rank, m.rot_dim, m.q_rank
+            st[p + "mix.dq"], st[p + "mix.dq.norm"] = rn(qr, W, s=W ** -0.5), 1 + rn(qr, s=0.1)
+            st[p + "mix.uq"] = rn(H * (dk + dr), qr, s=qr ** -0.5)
+            st[p + "mix.dkv"], st[p + "mix.dkv.norm"] = rn(rk + dr, W, s=W ** -0.5), 1 + rn(rk, s=0.1)
+            st[p + "mix.uk"], st[p + "mix.uv"] = rn(H * dk, rk, s=rk ** -0.5), rn(H * dv, rk, s=rk ** -0.5)
+            st[p + "mix.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
+        else:
+            G, sd = m.kv_heads, m.ssd
+            st[p + "mix.left.q"], st[p + "mix.left.k"] = rn(H * dk, W, s=W ** -0.5), rn(G * dk, W, s=W ** -0.5)
+            st[p + "mix.left.v"] = rn(G * dv, W, s=W ** -0.5)
+            st[p + "mix.left.q.norm"], st[p + "mix.left.k.norm"] = 1 + rn(H * dk, s=0.1), 1 + rn(G * dk, s=0.1)
+            st[p + "mix.left.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
+            st[p + "mix.right.in"] = rn(2 * sd.inner + 2 * sd.groups * sd.state + sd.heads, W, s=W ** -0.5)
+            st[p + "mix.right.conv"], st[p + "mix.right.conv.b"] = rn(sd.conv_channels, sd.taps, s=0.5), rn(sd.conv_channels, s=0.1)
+            st[p + "mix.right.dt_bias"], st[p + "mix.right.A_log"] = rn(sd.heads, s=0.5) - 1.0, rn(sd.heads, s=0.5) - 1.0
+            st[p + "mix.right.D"], st[p + "mix.right.norm"] = 1 + rn(sd.heads, s=0.2), 1 + rn(sd.inner, s=0.1)
+            st[p + "mix.right.o"] = rn(W, sd.inner, s=sd.inner ** -0.5)
+        ex = l.experts
+        if ex is not None:
+            st[p + "norm2"], st[p + "mlp.router"] = 1 + rn(W, s=0.1), rn(ex.experts, W, s=W ** -0.5)
+            for e in range(ex.experts):
+                st[p + f"mlp.e{e}.gate"], st[p + f"mlp.e{e}.up"] = rn(ex.ff, W, s=W ** -0.5), rn(ex.ff, W, s=W ** -0.5)
+                st[p + f"mlp.e{e}.down"] = rn(W, ex.ff, s=ex.ff ** -0.5)
     return st
 
 
