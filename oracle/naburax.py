@@ -273,7 +273,7 @@ def random_tensors(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
         if mlp:
             F, E = mlp["expert"]["ff"], mlp["router"]["experts"]
             t[p + "norm2"] = rn(Wd, s=0.1, mean=1.0)
-            t[p + "mlp.router"] = rn(E, Wd, s=1.0)
+            t[p + "mlp.router"] = rn(E, Wd, s=Wd ** -0.5)   # (logits of order one: no saturated, tied scores)
             for e in range(E):
                 t[p + f"mlp.e{e}.gate"], t[p + f"mlp.e{e}.up"] = rn(F, Wd, s=Wd ** -0.5), rn(F, Wd, s=Wd ** -0.5)
                 t[p + f"mlp.e{e}.down"] = rn(Wd, F, s=F ** -0.5)

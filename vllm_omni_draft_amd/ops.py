@@ -1182,3 +1182,144 @@ def relu_mul_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     _lib.check(_lib.load().sd_relu_mul_rows(_p(gate), _p(up), gate.shape[1], _p(out), gate.shape[0],
                                             gate.shape[1], _stream()), "sd_relu_mul_rows")
     return out
+
+
+# ---------------------------------------------------------------- mechanisms of hybrid layer-list models
+def embed_hashed(tokens, table, scale=1.0, prev_tokens=None, bigram=None, mul_prev=0, mul_cur=0,
+                 bf16_copy=False):
+    """table[tokens] * scale (+ bigram[(prev * mul_prev + tok * mul_cur) mod buckets], the table's
+    last row where prev_tokens is negative) as f32 [rows, W]."""
+    _need(tokens, torch.int32, "tokens")
+    n, W = tokens.numel(), table.shape[1]
+    x = torch.empty(n, W, dtype=torch.float32, device=table.device)
+    x_b = torch.empty(n, W, dtype=torch.bfloat16, device=table.device) if bf16_copy else None
+    _lib.check(_lib.load().sd_embed_hashed(_p(tokens), _p(prev_tokens), _p(table), _p(bigram), _wkind(table, "table"),
+                                           float(scale), bigram.shape[0] - 1 if bigram is not None else 0,
+                                           int(mul_prev), int(mul_cur), _p(x), _p(x_b), n, W, table.shape[0],
+                                           _stream()), "sd_embed_hashed")
+    return (x, x_b) if bf16_copy else x
+
+
+def rmsnorm_parts(x, w, eps, parts=1, gate=None, round_bf16=False, bf16_copy=False):
+    """x f32 [rows, width] in `parts` equal parts, each divided by its root mean square, times w
+    (or None); gate: x * silu(gate) is what gets normed."""
+    _f32(x, "x")
+    n, width = x.shape
+    out = torch.empty_like(x)
+    out_b = torch.empty_like(x, dtype=torch.bfloat16) if bf16_copy else None
+    _lib.check(_lib.load().sd_rmsnorm_parts(_p(x), width, _p(gate), gate.shape[1] if gate is not None else 0, _p(w),
+                                            _wkind(w, "w") if w is not None else 1, float(eps), _p(out), width,
+                                            _p(out_b), width, n, width, int(parts), int(round_bf16), _stream()),
+               "sd_rmsnorm_parts")
+    return (out, out_b) if bf16_copy else out
+
+
+def rope_rows(x, row_pos, heads, head_stride, offset, rot_dims, inv_freq, mag=1.0, layout=1) -> None:
+    """In place on x f32 [rows, ld]: see sd_rope_rows."""
+    _f32(x, "x")
+    _lib.check(_lib.load().sd_rope_rows(_p(x), x.shape[1], _p(row_pos), x.shape[0], heads, head_stride, offset,
+                                        rot_dims, layout, _p(inv_freq), float(mag), _stream()), "sd_rope_rows")
+
+
+def cache_append(k, v, k_cache, v_cache, row_pos, row_slot, block_tables, G, dk, dv) -> None:
+    _f32(k, "k")
+    _lib.check(_lib.load().sd_cache_append(_p(k), k.shape[1], _p(v), v.shape[1] if v is not None else 0, _p(k_cache),
+                                           _p(v_cache), int(k_cache.dtype == torch.float32), _p(row_pos),
+                                           _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, k.shape[0],
+                                           G, dk, dv, _stream()), "sd_cache_append")
+
+
+def window_softmax_attention(q, k_cache, v_cache, row_pos, row_slot, block_tables, H, G, dk, dv, window,
+                             keep_first, scale) -> torch.Tensor:
+    """q f32 [rows, H*dk]; caches [pages, G, PAGE, dk | dv]; v_cache None: values are the first dv
+    channels of the key rows.  Returns f32 [rows, H*dv]."""
+    _f32(q, "q")
+    out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().sd_window_softmax_attention(
+        _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(row_pos),
+        _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0], H, G, dk, dv, int(window),
+        int(keep_first), float(scale), _p(out), None, _stream()), "sd_window_softmax_attention")
+    return out
+
+
+def matmul_rows_batched(x, w) -> torch.Tensor:
+    """x f32 [M, B, K], w [B, N, K] -> f32 [M, B, N]: product b uses w[b]."""
+    _f32(x, "x")
+    M, B, K = x.shape
+    N = w.shape[1]
+    y = torch.empty(M, B, N, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().sd_matmul_rows_batched(_p(x), B * K, K, _p(w), _wkind(w, "w"), N * K, _p(y), B * N, N,
+                                                  None, M, N, K, B, _stream()), "sd_matmul_rows_batched")
+    return y
+
+
+def causal_conv_rows(x, w, b, conv_state, row_pos, row_slot, entries, act=True) -> torch.Tensor:
+    """x f32 [rows, C], w [C, taps], b [C] or None, conv_state f32 [slots, taps-1, C] (moved on)."""
+    _f32(x, "x")
+    _f32(conv_state, "conv_state")
+    out = torch.empty_like(x)
+    C_, taps = w.shape
+    _lib.check(_lib.load().sd_causal_conv_rows(_p(x), C_, _p(w), _p(b), _wkind(w, "w"), _p(conv_state), _p(row_pos),
+                                               _p(row_slot), _p(entries), entries.shape[0], _p(out), C_, x.shape[0],
+                                               C_, taps, int(act), _stream()), "sd_causal_conv_rows")
+    return out
+
+
+def ssd_steps(dt, dt_bias, a_log):
+    """(softplus(dt + dt_bias), exp(-exp(a_log) * that)) for dt f32 [rows, H]."""
+    _f32(dt, "dt")
+    step, decay = torch.empty_like(dt), torch.empty_like(dt)
+    _lib.check(_lib.load().sd_ssd_steps(_p(dt), dt.shape[1], _p(dt_bias), _p(a_log), _wkind(dt_bias, "dt_bias"),
+                                        _p(step), _p(decay), dt.shape[0], dt.shape[1], _stream()), "sd_ssd_steps")
+    return step, decay
+
+
+def decay_scan_rows(q, k, v, decay, k_scale, skip, state, entries, H, Gq, dk, dv) -> torch.Tensor:
+    """q, k f32 [rows, Gq*dk], v [rows, H*dv], decay / k_scale [rows, H], skip [H] or None,
+    state f32 [slots, H, dk, dv] (updated)."""
+    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (decay, "decay"), (state, "state")):
+        _f32(t, nm)
+    buf = torch.cat([q, k], dim=1).contiguous()
+    out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().sd_decay_scan_rows(buf.data_ptr(), buf.data_ptr() + 4 * Gq * dk, buf.shape[1], _p(v),
+                                              v.shape[1], _p(decay), _p(k_scale), _p(skip),
+                                              _wkind(skip, "skip") if skip is not None else 1, _p(state),
+                                              _p(entries), entries.shape[0], _p(out), H, Gq, dk, dv, _stream()),
+               "sd_decay_scan_rows")
+    return out
+
+
+def moe_route(logits, top, score="sigmoid", renorm=False):
+    """(chosen experts int32 [rows, top], their weights f32 [rows, top])."""
+    _f32(logits, "logits")
+    n, E = logits.shape
+    sel_e = torch.empty(n, top, dtype=torch.int32, device=logits.device)
+    sel_w = torch.empty(n, top, dtype=torch.float32, device=logits.device)
+    _lib.check(_lib.load().sd_moe_route(_p(logits), E, _p(sel_e), _p(sel_w), n, E, top,
+                                        {"sigmoid": 0, "softmax": 1}[score], int(renorm), _stream()), "sd_moe_route")
+    return sel_e, sel_w
+
+
+def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True) -> torch.Tensor:
+    """x f32 [rows, W]; w_gate_up [E, 2F, W], w_down [E, W, F]; returns f32 [rows, top, W]: every
+    chosen expert's result."""
+    _f32(x, "x")
+    n, W = x.shape
+    top, E, F = sel_e.shape[1], w_gate_up.shape[0], w_down.shape[2]
+    lib = _lib.load()
+    nb = int(lib.sd_moe_experts_scratch_bytes(n, top, E, F, W))
+    scratch = torch.empty(nb, dtype=torch.uint8, device=x.device)
+    out = torch.empty(n, top, W, dtype=torch.float32, device=x.device)
+    _lib.check(lib.sd_moe_experts(_p(x), W, _p(sel_e), _p(sel_w), _p(w_gate_up), _p(w_down), _wkind(w_down, "w_down"),
+                                  _p(out), n, top, E, F, W, int(scale_input), 0, _p(scratch), nb, _stream()),
+               "sd_moe_experts")
+    return out
+
+
+def postnorm_residual(x, a, w, eps, n_a=1, sa=1.0, b=None, sb=0.0) -> None:
+    """x += rms_norm(sa * (sum of each row's n_a rows of a) + sb * b) * w, in place."""
+    _f32(x, "x")
+    _f32(a, "a")
+    _lib.check(_lib.load().sd_postnorm_residual(_p(x), _p(a), int(n_a), float(sa), _p(b), float(sb), _p(w),
+                                                _wkind(w, "w"), float(eps), None, x.shape[0], x.shape[1], _stream()),
+               "sd_postnorm_residual")
