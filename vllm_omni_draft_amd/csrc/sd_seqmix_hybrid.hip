@@ -743,6 +743,122 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
   }
 }
 
+// ---- the same two products on the matrix cores (bf16 weights, K a multiple of 32).  A workgroup
+// takes one tile of kMoeBM assignment rows; its rows are staged in LDS as bf16 in chunks of
+// kMfKC columns, every wave reads its weight fragments straight from the row-major matrices
+// (a lane's 8 consecutive k of one weight row are 16 contiguous bytes).  16x16x32 tiles: operand
+// lane l holds row l%16, k-block l/16; result lane l holds rows 4*(l/16)..+3 of column l%16.
+constexpr int kMfKC = 512;
+constexpr int kMfLd = kMfKC + 8;   // LDS row stride in bf16: 16 rows at one k fall into distinct banks
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// act[a, n] (bf16) = silu(s * gate) * (s * up); a wave owns 16 columns of gate and of up.
+__global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
+    const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wgu,
+    bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
+  if ((int)blockIdx.y >= n_tiles[0]) return;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
+  __shared__ int arow[kMoeBM];
+  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
+  const int n = blockIdx.x * 64 + wave * 16 + lr;
+  const int nc = n < F ? n : F - 1;
+  const bf16_t* wg = Wgu + ((size_t)e * 2 * F + nc) * K + 8 * kq;
+  const bf16_t* wu = wg + (size_t)F * K;
+  if (tid < kMoeBM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  f32x4 ag[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, au[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
+    const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
+    __syncthreads();
+    for (int idx = tid; idx < kMoeBM * (kc / 4); idx += 256) {
+      const int m = idx / (kc / 4), k4 = (idx % (kc / 4)) * 4;
+      const int a = arow[m];
+      bf16x4 v = {0, 0, 0, 0};
+      if (a >= 0) {
+        const float* xr = X + (size_t)(a / top) * ldx + kc0 + k4;
+        v = bf16x4{(bf16_t)xr[0], (bf16_t)xr[1], (bf16_t)xr[2], (bf16_t)xr[3]};
+      }
+      *reinterpret_cast<bf16x4*>(xs + m * kMfLd + k4) = v;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int k0 = 0; k0 < kc; k0 += 32) {
+      const bf16x8 fg = *reinterpret_cast<const bf16x8*>(wg + kc0 + k0);
+      const bf16x8 fu = *reinterpret_cast<const bf16x8*>(wu + kc0 + k0);
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(xs + lr * kMfLd + k0 + 8 * kq);
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(xs + (16 + lr) * kMfLd + k0 + 8 * kq);
+      ag[0] = mfma16(a0, fg, ag[0]);
+      ag[1] = mfma16(a1, fg, ag[1]);
+      au[0] = mfma16(a0, fu, au[0]);
+      au[1] = mfma16(a1, fu, au[1]);
+    }
+  }
+  if (n >= F) return;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int a = arow[mt * 16 + 4 * kq + i];
+      if (a < 0) continue;
+      const float sc = scale_input ? sel_w[a] : 1.f;
+      act[(size_t)a * F + n] = (bf16_t)(silu_f(sc * ag[mt][i]) * (sc * au[mt][i]));
+    }
+}
+
+// out[a, n] = down_e act[a]; a wave owns 32 columns.
+__global__ __launch_bounds__(256) void moe_down_mfma_kernel(
+    const bf16_t* __restrict__ act, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wd,
+    float* __restrict__ out, int N, int K, int scale_input) {
+  if ((int)blockIdx.y >= n_tiles[0]) return;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
+  __shared__ int arow[kMoeBM];
+  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * 128 + wave * 32 + lr, n1 = n0 + 16;
+  const bf16_t* w0 = Wd + ((size_t)e * N + (n0 < N ? n0 : N - 1)) * K + 8 * kq;
+  const bf16_t* w1 = Wd + ((size_t)e * N + (n1 < N ? n1 : N - 1)) * K + 8 * kq;
+  if (tid < kMoeBM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  f32x4 acc[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+  for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
+    const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
+    __syncthreads();
+    for (int idx = tid; idx < kMoeBM * (kc / 8); idx += 256) {
+      const int m = idx / (kc / 8), k8 = (idx % (kc / 8)) * 8;
+      const int a = arow[m];
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (a >= 0) v = *reinterpret_cast<const bf16x8*>(act + (size_t)a * K + kc0 + k8);
+      *reinterpret_cast<bf16x8*>(xs + m * kMfLd + k8) = v;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int k0 = 0; k0 < kc; k0 += 32) {
+      const bf16x8 f0 = *reinterpret_cast<const bf16x8*>(w0 + kc0 + k0);
+      const bf16x8 f1 = *reinterpret_cast<const bf16x8*>(w1 + kc0 + k0);
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(xs + lr * kMfLd + k0 + 8 * kq);
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(xs + (16 + lr) * kMfLd + k0 + 8 * kq);
+      acc[0][0] = mfma16(a0, f0, acc[0][0]);
+      acc[1][0] = mfma16(a1, f0, acc[1][0]);
+      acc[0][1] = mfma16(a0, f1, acc[0][1]);
+      acc[1][1] = mfma16(a1, f1, acc[1][1]);
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int a = arow[mt * 16 + 4 * kq + i];
+      if (a < 0) continue;
+      const float sc = scale_input ? 1.f : sel_w[a];
+      if (n0 < N) out[(size_t)a * N + n0] = sc * acc[mt][0][i];
+      if (n1 < N) out[(size_t)a * N + n1] = sc * acc[mt][1][i];
+    }
+}
+
 struct MoeScratch {
   size_t cnt, n_tiles, perm, tiles, act, total;
 };
@@ -1033,6 +1149,15 @@ extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_ex
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_kernel<float><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
                                                                          (const float*)w_down, out, W, F, scale_input);
+  } else if (W % 32 == 0 && F % 32 == 0 && sd_aligned16(w_gate_up) && sd_aligned16(w_down)) {
+    // (act holds n * F floats: its first half serves as the bf16 activations)
+    bf16_t* act_b = (bf16_t*)act;
+    moe_gate_up_mfma_kernel<<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
+                                                                          (const bf16_t*)w_gate_up, act_b, top, F, W,
+                                                                          scale_input);
+    SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
+    moe_down_mfma_kernel<<<dim3((W + 127) / 128, tiles_y), 256, 0, st>>>(act_b, perm, tiles, n_tiles, sel_weight,
+                                                                         (const bf16_t*)w_down, out, W, F, scale_input);
   } else {
     moe_gate_up_kernel<bf16_t><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
                                                                              (const bf16_t*)w_gate_up, act, top, F, W, scale_input, 1);
