@@ -102,12 +102,14 @@ def parse():
     ap.add_argument("--tp-draft", choices=["replicated", "sharded"], default="replicated",
                     help="the draft whole on every rank (no exchange in its passes), or sharded "
                          "like the target with a vocabulary-parallel head")
-    ap.add_argument("--family", choices=["spec", "puguzen"], default="spec",
+    ap.add_argument("--family", choices=["spec", "puguzen", "naburax"], default="spec",
                     help="spec: the headline speculative-decoding workload (default).  puguzen: prefill and "
                          "decode throughput of the Puguzen decoder family (recurrent and windowed layers) at "
                          "layer sizes of real models, beside a Llama-style decoder of equal size, with the "
-                         "time and memory traffic of its own kernels")
-    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen: sizes to run")
+                         "time and memory traffic of its own kernels.  naburax: the same for the Naburax "
+                         "family (latent attention, attention beside a state-space recurrence, routed "
+                         "experts), beside the Puguzen family at equal size")
+    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen / naburax: sizes to run")
     return ap.parse_args()
 
 
@@ -797,9 +799,170 @@ def main_seq_family(args):
     print(json.dumps({"metric": "puguzen_family_throughput", "unit": "tokens/s", "dtype": "bf16",
                       "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
 
+# ---------------------------------------------------------------------------------------------
+# --family naburax
+NAB_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, q_rank=512, s_heads=16, experts=8, top=2, eff=1024),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, q_rank=768, s_heads=32, experts=16, top=2, eff=2048),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, q_rank=1536, s_heads=64, experts=16, top=2, eff=4096),
+}
+NAB_KV_RANK, NAB_ROT, NAB_STATE, NAB_SVDIM, NAB_KEEP = 512, 64, 128, 64, 4
+F32_VALU_PEAK_TFLOPS = 157.0   # MI355X vector f32 peak
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
+
+
+def _nab_config(sz):
+    from vllm_omni_draft_amd.config import ExpertsSpec, MixerSpec, SeqLayerSpec, SeqModelConfig, SsdSpec
+    H, G, D = sz["heads"], sz["kv_heads"], SEQ_HEAD
+    lat = MixerSpec("latent_attention", H, D, D, q_rank=sz["q_rank"], kv_rank=NAB_KV_RANK, rot_dim=NAB_ROT,
+                    rot_dims=NAB_ROT, rot_base=1e6, rot_layout="interleaved",
+                    rot_scaling={"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0},
+                    scale=(D + NAB_ROT) ** -0.5, window=SEQ_WINDOW)
+    par = MixerSpec("parallel", H, D, D, kv_heads=G, scale=D ** -0.5, window=SEQ_WINDOW, keep_first=NAB_KEEP,
+                    ssd=SsdSpec(heads=sz["s_heads"], vdim=NAB_SVDIM, state=NAB_STATE, groups=1, taps=4,
+                                norm_groups=1), left_scale=0.5, right_scale=0.5)
+    ex = ExpertsSpec(sz["experts"], sz["top"], sz["eff"])
+    cfg = SeqModelConfig("naburax", sz["width"], SEQ_VOCAB, [SeqLayerSpec(m, 0, ex) for m in (lat, par, lat, par)],
+                         name="naburax-bench", block="postnorm", embed_scale=1.0,
+                         bigram={"buckets": 65521, "mul_prev": 31, "mul_cur": 17}, tied_head=False, logit_scale=1.0)
+    cfg.validate()
+    return cfg
+
+
+def _run_seq_engine(cfg, device, P, B, steps, warm):
+    """Prefill time of one P-token prompt and time of `steps` decoding steps of B sequences."""
+    from vllm_omni_draft_amd import weights
+    from vllm_omni_draft_amd.seq_engine import SeqEngine, SeqEngineConfig
+    w = weights.seq_from_state_dict(cfg, weights.seq_random_state(cfg, 0), device, torch.bfloat16)
+    g = torch.Generator().manual_seed(7)
+    prompts = [torch.randint(0, cfg.vocab, (P,), generator=g).tolist() for _ in range(B)]
+    eng = SeqEngine(w, SeqEngineConfig(max_seqs=B, max_tokens=B * (P + steps + warm + 64), max_rows=2048,
+                                       max_seq_len=P + steps + warm + 64))
+    eng.step([("warm", prompts[0][:300], [299])])
+    eng.finish("warm")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.step([("s0", prompts[0], [P - 1])])
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    for i in range(1, B):
+        eng.step([(f"s{i}", prompts[i], [P - 1])])
+    toks = [1] * B
+
+    def decode(n):
+        nonlocal toks
+        for _ in range(n):
+            lg = eng.step([(f"s{i}", [toks[i]], [0]) for i in range(B)])
+            toks = lg.argmax(-1).tolist()
+    decode(warm)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    decode(steps)
+    torch.cuda.synchronize()
+    decode_s = time.perf_counter() - t0
+    nbytes = w.nbytes()
+    del eng, w
+    torch.cuda.empty_cache()
+    return {"weight_bytes": nbytes, "prefill_tokens_per_s": round(P / prefill_s, 1),
+            "decode_tokens_per_s": round(B * steps / decode_s, 1), "decode_ms_per_step": round(decode_s / steps * 1e3, 3)}
+
+
+def nab_kernel_rooflines(cfg, device, ctx, rows):
+    """The family's own kernels alone at `rows` token rows of one sequence that ends at position
+    ctx: time, the bytes and the floating-point operations each needs at least, and how far that
+    puts it from the nearer of its two rooflines (HBM, or the f32 vector / bf16 matrix peak)."""
+    from vllm_omni_draft_amd import ops
+    lat = next(l.mixer for l in cfg.layers if l.mixer.kind == "latent_attention")
+    par = next(l.mixer for l in cfg.layers if l.mixer.kind == "parallel")
+    ex, W = cfg.layers[0].experts, cfg.width
+    g = torch.Generator(device="cpu").manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g).to(device)
+    pages = -(-ctx // ops.PAGE)
+    tables = torch.arange(pages, dtype=torch.int32, device=device).view(1, -1)
+    pos = torch.arange(ctx - rows, ctx, dtype=torch.int32, device=device)
+    slot = torch.zeros(rows, dtype=torch.int32, device=device)
+    keys = sum(min(int(p) + 1, lat.window) for p in pos.tolist())     # (row, key) pairs inside the window
+    span = min(ctx, lat.window + rows - 1)                            # distinct keys read
+    out = []
+    # latent attention: one cached row per token is key and value
+    H, de, rk = lat.heads, lat.kv_rank + lat.rot_dim, lat.kv_rank
+    kc = (torch.randn(pages, 1, ops.PAGE, de, generator=g) * 0.3).to(torch.bfloat16).to(device)
+    q = rn(rows, H * de)
+    us = _events(lambda: ops.window_softmax_attention(q, kc, None, pos, slot, tables, H, 1, de, rk, lat.window, 0,
+                                                      lat.scale), 5)
+    out.append(("window_softmax_attention (latent rows)", us, 2 * de * span + 4 * rows * H * (de + rk),
+                2.0 * keys * H * (de + rk), F32_VALU_PEAK_TFLOPS))
+    # grouped-query attention with kept first tokens
+    H, G, D = par.heads, par.kv_heads, par.dim
+    kc2 = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    vc2 = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    q2 = rn(rows, H * D)
+    us = _events(lambda: ops.window_softmax_attention(q2, kc2, vc2, pos, slot, tables, H, G, D, D, par.window,
+                                                      par.keep_first, par.scale), 5)
+    out.append(("window_softmax_attention (grouped heads)", us, G * 2 * D * 2 * span + 8 * rows * H * D,
+                2.0 * keys * H * 2 * D, F32_VALU_PEAK_TFLOPS))
+    # state-space scan
+    sd = par.ssd
+    Hs, N_, Pv = sd.heads, sd.state, sd.vdim
+    qs, ks, vs = rn(rows, N_), rn(rows, N_) * N_ ** -0.5, rn(rows, Hs * Pv)
+    dec, stp = torch.rand(rows, Hs, generator=g).to(device) * 0.1 + 0.9, torch.rand(rows, Hs, generator=g).to(device)
+    state = torch.zeros(1, Hs, N_, Pv, device=device)
+    ent = torch.tensor([[0, 0, rows, 1]], dtype=torch.int32, device=device)
+    skip = torch.ones(Hs, device=device)
+    us = _events(lambda: ops.decay_scan_rows(qs, ks, vs, dec, stp, skip, state, ent, Hs, 1, N_, Pv), 5)
+    out.append(("decay_scan_rows", us, 4 * (rows * (2 * N_ + 2 * Hs * Pv + 2 * Hs) + 2 * Hs * N_ * Pv),
+                rows * Hs * N_ * Pv * 5.0, F32_VALU_PEAK_TFLOPS))
+    # routed experts (grouping, gate / up, down)
+    E, top, F = ex.experts, ex.top, ex.ff
+    x = rn(rows, W)
+    gu = (torch.randn(E, 2 * F, W, generator=g) * W ** -0.5).to(torch.bfloat16).to(device)
+    dn = (torch.randn(E, W, F, generator=g) * F ** -0.5).to(torch.bfloat16).to(device)
+    sel_e = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(rows)]).to(torch.int32).to(device)
+    sel_w = torch.rand(rows, top, generator=g).to(device)
+    us = _events(lambda: ops.moe_experts(x, sel_e, sel_w, gu, dn), 5)
+    used = min(E, rows * top)
+    out.append(("moe_experts", us, 2 * used * 3 * F * W + 4 * rows * W * (1 + top) + 2 * rows * top * F * 2,
+                2.0 * rows * top * 3 * F * W, BF16_MFMA_PEAK_TFLOPS))
+    res = []
+    for name, us, nbytes, flops, peak in out:
+        floor_us = max(nbytes / (HBM_PEAK_GBS * 1e3), flops / (peak * 1e6))
+        res.append({"kernel": name, "rows": rows, "ctx": ctx, "avg_us": round(us, 2), "min_bytes": int(nbytes),
+                    "flops": int(flops), "achieved_gbs": round(nbytes / us * 1e-3, 1),
+                    "achieved_tflops": round(flops / us * 1e-6, 2), "roofline_us": round(floor_us, 2),
+                    "times_roofline": round(us / floor_us, 1)})
+    return res
+
+
+def main_nab_family(args):
+    """Prefill and decode throughput of the Naburax family beside the Puguzen family at equal
+    width, heads and active feed-forward width (both bf16, seeded random weights), one JSON line."""
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (there is no CPU path)")
+    device = torch.device("cuda", 0)
+    P, B, steps, warm = args.prompt_len, 4, args.steps, args.warmup
+    results = []
+    for name in args.seq_sizes.split(","):
+        sz = NAB_SIZES[name]
+        cfg = _nab_config(sz)
+        mine = _run_seq_engine(cfg, device, P, B, steps, warm)
+        kern = nab_kernel_rooflines(cfg, device, P, 1) + nab_kernel_rooflines(cfg, device, P, min(P, 1024))
+        pz = dict(SEQ_SIZES[name], ff=sz["top"] * sz["eff"])
+        pcfg = _seq_config(pz)
+        other = _run_seq_engine(pcfg, device, P, B, steps, warm)
+        like = seq_kernel_rooflines(pcfg, device, P, 1) + seq_kernel_rooflines(pcfg, device, P, min(P, 1024))
+        results.append({"size": name, **sz, "layers": [l.mixer.kind for l in cfg.layers], "head_dim": SEQ_HEAD,
+                        "kv_rank": NAB_KV_RANK, "rot_dim": NAB_ROT, "state": NAB_STATE, "window": SEQ_WINDOW,
+                        "keep_first": NAB_KEEP, "prompt_len": P, "decode_batch": B, "naburax": mine,
+                        "puguzen_equal_size": other, "kernels": kern, "puguzen_kernels": like})
+    print(json.dumps({"metric": "naburax_family_throughput", "unit": "tokens/s", "dtype": "bf16",
+                      "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
+
 
 def main():
     args = parse()
+    if args.family == "naburax":
+        main_nab_family(args)
+        return
     if args.family == "puguzen":
         main_seq_family(args)
         return

@@ -1152,13 +1152,19 @@ int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, vo
  * head h reads kv head h / (H/G).  v_cache == NULL: a value row is the first dv channels of its
  * key row (latent attention: keys and values share one cached row).  Keys are taken in the
  * order kept tokens, then window, in tiles of 256 with a running maximum; dv <= 512.
- * out_bf16 (or NULL): the same as bf16.                                                     */
+ * out_bf16 (or NULL): the same as bf16.  scratch (may be NULL):
+ * sd_window_softmax_attention_scratch_bytes(n_rows, ..., max_blocks * page) bytes let a batch of
+ * few rows cut each row's keys into tiles of 64 that run as workgroups of their own (a second
+ * kernel merges a row's tiles in order); 0 bytes means that no such cut would be made.       */
+size_t sd_window_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window,
+                                                 int keep_first, int max_ctx);
 int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache,
                                 const void* v_cache, int cache_f32, const int32_t* row_pos,
                                 const int32_t* row_slot, const int32_t* block_tables,
                                 int max_blocks, int page, int n_rows, int H, int G, int dk, int dv,
                                 int window, int keep_first, float scale, float* out,
-                                void* out_bf16, sd_stream_t stream);
+                                void* out_bf16, void* scratch, size_t scratch_bytes,
+                                sd_stream_t stream);
 /* y[z][M, N] = x[z][M, K] w[z][N, K]^T for z < batch: x + z*bx (row stride ldx), w + z*bw,
  * y + z*by (row stride ldy); y_bf16 (or NULL) laid out as y.                                */
 int sd_matmul_rows_batched(const float* x, int64_t ldx, int64_t bx, const void* w, int w_f32,
@@ -1189,6 +1195,12 @@ int sd_decay_scan_rows(const float* q, const float* k, int64_t ldqk, const float
  * sel_weight [rows, top], weights divided by their sum when renorm.                          */
 int sd_moe_route(const float* logits, int64_t ld, int32_t* sel_expert, float* sel_weight,
                  int n_rows, int E, int top, int score_kind, int renorm, sd_stream_t stream);
+/* The router's product and the choice in one launch: logits[r, e] = x[r] . w_router[e] (x [rows, K]
+ * row stride ldx, rounded to bf16 values when the weights are bf16; w_router [E, K]; logits
+ * [rows, E] or NULL), then as sd_moe_route.                                                  */
+int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_router, int w_f32, float* logits,
+                      int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
+                      int score_kind, int renorm, sd_stream_t stream);
 /* Bytes of scratch sd_moe_experts needs.                                                   */
 size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W);
 /* out[r*top + j] = down_e(act(gate_e u) * (up_e u)) for e = sel_expert[r, j], u = sel_weight *

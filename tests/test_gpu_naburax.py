@@ -280,6 +280,16 @@ def test_window_softmax_attention_many_keys(cdt):
                                       torch.tensor(rows), 0.5, window, keep)
     assert rel(out, want.reshape(4, -1)) < 3e-6
     assert rel(out[0, :dv], v[70].double()) < 1e-3     # that key takes all the weight
+    # few rows have their keys cut over workgroups and merged; many rows, or no scratch, take them in one sweep
+    whole = ops.window_softmax_attention(dev(q), kc, vc, i32(rows), i32([0] * 4), bt, H, G, dk, dv, window, keep, 0.5,
+                                         split=False)
+    assert rel(whole, want.reshape(4, -1)) < 3e-6 and rel(whole, out) < 2e-6
+    many = list(range(600, 700))
+    q2 = torch.randn(100, H * dk, generator=g)
+    out2 = ops.window_softmax_attention(dev(q2), kc, vc, i32(many), i32([0] * 100), bt, H, G, dk, dv, window, keep, 0.5)
+    one = ops.window_softmax_attention(dev(q2[37:38]), kc, vc, i32(many[37:38]), i32([0]), bt, H, G, dk, dv, window,
+                                       keep, 0.5)
+    assert rel(one[0], out2[37]) < 2e-6
 
 
 @pytest.mark.parametrize("M,B,N_,K", [(1, 3, 7, 5), (5, 2, 130, 24), (40, 6, 16, 136)])
@@ -364,7 +374,7 @@ def test_routed_experts(E, top, F, W, rows, wdt):
     x = torch.randn(rows, W, generator=g)
     if wdt == torch.bfloat16:
         x = x.to(wdt).float()
-    Wt = {"router": torch.randn(E, W, generator=g).to(wdt)}
+    Wt = {"router": (torch.randn(E, W, generator=g) * W ** -0.5).to(wdt)}    # (logits of order one: no tied scores)
     for e in range(E):
         Wt[f"e{e}.gate"], Wt[f"e{e}.up"] = (torch.randn(F, W, generator=g) * W ** -0.5).to(wdt), \
             (torch.randn(F, W, generator=g) * W ** -0.5).to(wdt)
@@ -382,6 +392,21 @@ def test_routed_experts(E, top, F, W, rows, wdt):
     # a row's results do not depend on the rows around it
     one = ops.moe_experts(dev(x[:1]), sel_e[:1].contiguous(), sel_w[:1].contiguous(), dev(gu), dev(dn))
     assert torch.equal(one[0], out[0])
+
+
+@pytest.mark.parametrize("E,K,top,wdt", [(5, 40, 3, torch.float32), (16, 1000, 2, torch.bfloat16), (130, 64, 7, torch.float32)])
+def test_router_product_and_choice_in_one_launch(E, K, top, wdt):
+    from vllm_omni_draft_amd import ops
+    g = torch.Generator().manual_seed(E)
+    x, w = torch.randn(9, K, generator=g), (torch.randn(E, K, generator=g) * K ** -0.5).to(wdt)
+    xr = x.to(torch.bfloat16).double() if wdt == torch.bfloat16 else x.double()
+    e, sw, logits = ops.moe_route_rows(dev(x), dev(w), top)
+    want = xr @ w.double().T
+    assert rel(logits, want) < 2e-6
+    tk = torch.topk(torch.sigmoid(want), top)
+    assert torch.equal(e.cpu().long(), tk.indices) and rel(sw, tk.values) < 1e-6
+    e1, sw1, l1 = ops.moe_route_rows(dev(x[4:5]), dev(w), top)          # a row alone: the same bits
+    assert torch.equal(l1[0], logits[4]) and torch.equal(e1[0], e[4]) and torch.equal(sw1[0], sw[4])
 
 
 def test_router_other_scores():

@@ -241,13 +241,15 @@ SIGNATURES = {
     "sd_rope_rows": (i32, [vp, i64, vp, i32, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
     "sd_rope_copy_rows": (i32, [vp, i64, i32, i32, vp, i64, i32, i32, vp, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
     "sd_cache_append": (i32, [vp, i64, vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
+    "sd_window_softmax_attention_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32, i32]),
     "sd_window_softmax_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32,
-                                          i32, C.c_float, vp, vp, vp]),
+                                          i32, C.c_float, vp, vp, vp, C.c_size_t, vp]),
     "sd_matmul_rows_batched": (i32, [vp, i64, i64, vp, i32, i64, vp, i64, i64, vp, i32, i32, i32, i32, vp]),
     "sd_causal_conv_rows": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, vp, i32, vp, i64, i32, i32, i32, i32, vp]),
     "sd_ssd_steps": (i32, [vp, i64, vp, vp, i32, vp, vp, i32, i32, vp]),
     "sd_decay_scan_rows": (i32, [vp, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, i32, vp, i32, i32, i32, i32, vp]),
     "sd_moe_route": (i32, [vp, i64, vp, vp, i32, i32, i32, i32, i32, vp]),
+    "sd_moe_route_rows": (i32, [vp, i64, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
     "sd_moe_experts_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
     "sd_moe_experts": (i32, [vp, i64, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_size_t, vp]),
     "sd_postnorm_residual": (i32, [vp, vp, i32, C.c_float, vp, C.c_float, vp, i32, C.c_float, vp, i32, i32, vp]),

@@ -661,10 +661,78 @@ __global__ void relu_mul_rows_kernel(const float* __restrict__ gate, const float
     out[(size_t)r * F + c] = (bf16_t)(fmaxf(gate[(size_t)r * ld + c], 0.f) * up[(size_t)r * ld + c]);
 }
 
+// The same product for at most 16 rows: a workgroup takes one row (held in LDS) and a block of
+// output columns, a thread owns one column and walks its weight row in 16-byte pieces, many in
+// flight.  Every output is summed over k in ascending order with the same fused multiply-adds
+// as matmul_rows_kernel: the same bits.
+constexpr int kSkinnyRows = 16;
+constexpr int kSkinnyLoads = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void matmul_skinny_kernel(
+    const float* __restrict__ X, int64_t ldx, const T* __restrict__ Wt, const float* __restrict__ bias,
+    float* __restrict__ Y, int64_t ldy, int N, int K, int round, int64_t bx, int64_t bw, int64_t by,
+    bf16_t* __restrict__ Yb, int vec) {
+  extern __shared__ float xs[];   // [K]
+  const int i = blockIdx.y;
+  X += (size_t)blockIdx.z * bx + (size_t)i * ldx;
+  Wt += (size_t)blockIdx.z * bw;
+  Y += (size_t)blockIdx.z * by + (size_t)i * ldy;
+  if (Yb) Yb += (size_t)blockIdx.z * by + (size_t)i * ldy;
+  for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = maybe_round(X[k], round);
+  __syncthreads();
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  const T* wr = Wt + (size_t)n * K;
+  float acc = 0.f;
+  constexpr int E = 16 / sizeof(T);
+  int k = 0;
+  if (vec) {
+    for (; k < K; k += kSkinnyLoads * E) {
+      u32x4 raw[kSkinnyLoads];
+#pragma unroll
+      for (int p = 0; p < kSkinnyLoads; ++p) {   // unguarded, on an address clamped into the row
+        const int kp = k + p * E < K ? k + p * E : K - E;
+        raw[p] = *reinterpret_cast<const u32x4*>(wr + kp);
+      }
+#pragma unroll
+      for (int p = 0; p < kSkinnyLoads; ++p) {
+        if (k + p * E < K) {
+          float wf[E];
+          if constexpr (sizeof(T) == 2) {
+            const bf16x8 v = __builtin_bit_cast(bf16x8, raw[p]);
+#pragma unroll
+            for (int e = 0; e < E; ++e) wf[e] = (float)v[e];
+          } else {
+            const f32x4 v = __builtin_bit_cast(f32x4, raw[p]);
+#pragma unroll
+            for (int e = 0; e < E; ++e) wf[e] = v[e];
+          }
+#pragma unroll
+          for (int e = 0; e < E; ++e) acc = fmaf(xs[k + p * E + e], wf[e], acc);
+        }
+      }
+    }
+  } else {
+    for (; k < K; ++k) acc = fmaf(xs[k], ld_f(wr + k), acc);
+  }
+  const float o = acc + (bias ? bias[n] : 0.f);
+  Y[n] = o;
+  if (Yb) Yb[n] = (bf16_t)o;
+}
+
 template <typename T>
 int launch_matmul(const float* X, const float* X2, int64_t ldx, const void* Wt, const float* bias, float* Y,
                   int64_t ldy, int M, int N, int K, int round, hipStream_t st, int batch = 1, int64_t bx = 0,
                   int64_t bw = 0, int64_t by = 0, bf16_t* Yb = nullptr) {
+  if (M <= kSkinnyRows && !X2 && N >= 64 && (size_t)K * sizeof(float) <= 48 * 1024) {
+    const int vec = (K * sizeof(T)) % 16 == 0 && (bw * sizeof(T)) % 16 == 0 && sd_aligned16(Wt);
+    const int nthr = N >= 4096 ? 256 : (N >= 1024 ? 128 : 64);   // few columns: more, smaller workgroups
+    dim3 grid((N + nthr - 1) / nthr, M, batch);
+    matmul_skinny_kernel<T><<<grid, nthr, (size_t)K * sizeof(float), st>>>(X, ldx, (const T*)Wt, bias, Y, ldy, N, K,
+                                                                           round, bx, bw, by, Yb, vec);
+    SD_CHECK_LAUNCH("sd_matmul_rows");
+    return SD_OK;
+  }
   if (M <= 16) {
     dim3 grid((N + 127) / 128, (M + 15) / 16, batch);
     matmul_rows_kernel<T, 16, 128, 2, 4><<<grid, 256, 0, st>>>(X, X2, ldx, (const T*)Wt, bias, Y, ldy, M, N, K, round,
@@ -973,6 +1041,8 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
       need(l.w_in_tiled, wr, c.total, W);
       need(l.w_o_tiled, wr, W, l.heads * l.vdim);
       up(hv, (size_t)l.heads * l.vdim);
+      up(attn, sd_window_softmax_attention_scratch_bytes(rows, l.heads, l.kind == SD_MIX_LATENT ? l.kv_rank : l.vdim,
+                                                         l.window, l.keep_first, max_ctx));
       if (l.kind == SD_MIX_LATENT) {
         up(pq, (size_t)l.heads * (l.dim + l.rot_dim));
         up(qe, (size_t)l.heads * (l.kv_rank + l.rot_dim));
@@ -1184,7 +1254,7 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
                                l.rot_dims, 1, l.inv_freq, l.rot_mag, stream));
     SQ_TRY(sd_window_softmax_attention(qe, (int64_t)H * de, l.k_cache, nullptr, f32, b.row_pos, b.row_slot,
                                        b.block_tables, b.max_blocks, b.page, R, H, 1, de, rk, l.window, 0,
-                                       l.score_scale, o, nullptr, stream));
+                                       l.score_scale, o, nullptr, base + w.attn, w.attn_bytes, stream));
     // a head's value expansion applied to its weighted latent
     SQ_TRY(sd_matmul_rows_batched(o, (int64_t)H * rk, rk, l.w_uv, f32, (int64_t)dv * rk, y, (int64_t)H * dv, dv,
                                   l.w_o_tiled ? yb : nullptr, R, dv, rk, H, stream));
@@ -1202,7 +1272,8 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
                            b.block_tables, b.max_blocks, b.page, R, G, dk, dv, stream));
     SQ_TRY(sd_window_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
                                        b.block_tables, b.max_blocks, b.page, R, H, G, dk, dv, l.window, l.keep_first,
-                                       l.score_scale, o, l.w_o_tiled ? yb : nullptr, stream));
+                                       l.score_scale, o, l.w_o_tiled ? yb : nullptr, base + w.attn, w.attn_bytes,
+                                       stream));
     SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, o, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
                       H * dv, wide_ws, w.wide_bytes, stream));
     // state-space recurrence: convolution + silu over x, B, C; step sizes; scan; gate, group norm
@@ -1227,8 +1298,7 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
     float* sel_w = (float*)(base + w.sel_w);
     float* dn = (float*)(base + w.dn);
     const int E = l.n_experts;
-    SQ_TRY(sd_matmul_rows(x, nullptr, W, l.w_router, f32, nullptr, rlog, E, R, E, W, stream));
-    SQ_TRY(sd_moe_route(rlog, E, sel_e, sel_w, R, E, l.top, 0, 0, stream));
+    SQ_TRY(sd_moe_route_rows(x, W, l.w_router, f32, rlog, sel_e, sel_w, R, E, W, l.top, 0, 0, stream));
     SQ_TRY(sd_moe_experts(x, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, E, l.expert_ff, W, 1, 0,
                           base + w.moe, w.moe_bytes, stream));
     SQ_TRY(sd_postnorm_residual(x, dn, l.top, 1.f, nullptr, 0.f, l.norm2_w, f32, eps, hb, R, W, stream));

@@ -128,7 +128,6 @@ __global__ void cache_append_kernel(const float* __restrict__ k, int64_t ldk, co
 }
 
 // ------------------------------------------------------------------ softmax window attention
-constexpr int kTile = 256;     // keys per tile
 constexpr int kLoads = 16;     // 16-byte pieces of a key row a thread has in flight
 
 template <typename T> struct Piece;
@@ -188,31 +187,36 @@ __device__ __forceinline__ void score_key(const KT* __restrict__ kr, const float
 }
 
 // One workgroup per (row, kv head, group of up to NH query heads of that kv head).  Per tile of
-// 256 keys: a thread per key scores it against the query heads (q in LDS); the tile's maximum
-// moves the running maximum and rescales what has been summed; then a wave per key, lanes over
-// value columns, adds the weighted value rows.  NC: value columns per lane (dv <= 64 * NC).
-template <typename T, int NH, int NC>
-__global__ __launch_bounds__(256) void window_softmax_attn_kernel(
+// blockDim.x keys: a thread per key scores it against the query heads (q in LDS); the tile's
+// maximum moves the running maximum and rescales what has been summed; then a wave per key, lanes
+// over value columns, adds the weighted value rows.  NC: value columns per lane (dv <= 64 * NC).
+// n_splits > 1 (few rows): workgroup (.., .., z) takes tile z / n_hgroups of the row's keys only
+// and leaves its maximum, its sum of weights and its unnormalised weighted values in part_ml /
+// part_acc; softmax_merge_kernel puts a row's tiles together in tile order.
+template <typename T, int NH, int NC, int NT>
+__global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
     const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     int v_row, const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
     const int32_t* __restrict__ block_tables, int max_blocks, int page, int H, int G, int dk, int dv, int window,
-    int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups) {
+    int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups, int n_splits,
+    float* __restrict__ part_acc, float* __restrict__ part_ml) {
   extern __shared__ float lds[];
-  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [kTile] cache row of the key
-  float* wt = reinterpret_cast<float*>(vat + kTile);                     // [NH][kTile]
-  float* qs = wt + NH * kTile;                                           // [NH][dk]
+  constexpr int nthr = NT, nw = NT >> 6;   // threads = keys per tile; waves
+  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [nthr] cache row of the key
+  float* wt = reinterpret_cast<float*>(vat + nthr);                      // [NH][nthr]
+  float* qs = wt + NH * nthr;                                            // [NH][dk]
   float* m_run = qs + NH * dk;                                           // [NH] running maximum
   float* l_run = m_run + NH;                                             // [NH] running sum
   float* corr = l_run + NH;                                              // [NH]
-  float* red = corr + NH;                                                // [4][dv]
+  float* red = corr + NH;                                                // [nw][dv]
   const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
-  const int hgroup = blockIdx.z;
+  const int hgroup = blockIdx.z % n_hgroups, split = blockIdx.z / n_hgroups;
   const int qh = H / G;
   const int h0 = g * qh + hgroup * NH;
   const int nh = qh - hgroup * NH < NH ? qh - hgroup * NH : NH;
   const int i = row_pos[r];
   const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
-  for (int c = tid; c < nh * dk; c += 256) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
+  for (int c = tid; c < nh * dk; c += nthr) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
   if (tid < NH) {
     m_run[tid] = -INFINITY;
     l_run[tid] = 0.f;
@@ -220,6 +224,8 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
   const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
   const int n_kept = keep_first < t_first ? keep_first : t_first;   // kept tokens that left the window
   const int total = n_kept + (i - t_first + 1);
+  const int key_lo = n_splits > 1 ? split * nthr : 0;
+  const int key_hi = n_splits > 1 ? (total < key_lo + nthr ? total : key_lo + nthr) : total;
   const bool vec = dk % Piece<T>::E == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
   const int wave = tid >> 6, lane = tid & 63;
   float acc[NH][NC];
@@ -228,13 +234,13 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
 #pragma unroll
     for (int m = 0; m < NC; ++m) acc[hq][m] = 0.f;
   __syncthreads();
-  for (int base = 0; base < total; base += kTile) {
+  for (int base = key_lo; base < key_hi; base += nthr) {
     const int idx = base + tid;
     {
       float s[NH];
 #pragma unroll
       for (int hq = 0; hq < NH; ++hq) s[hq] = 0.f;
-      if (idx < total) {
+      if (idx < key_hi) {
         const int j = idx < n_kept ? idx : t_first + (idx - n_kept);
         const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
         score_key<T, NH>(k_cache + at * dk, qs, dk, nh, vec, s);
@@ -242,12 +248,12 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       }
 #pragma unroll
       for (int hq = 0; hq < NH; ++hq)
-        if (hq < nh) wt[hq * kTile + tid] = idx < total ? s[hq] * scale : -INFINITY;
+        if (hq < nh) wt[hq * nthr + tid] = idx < key_hi ? s[hq] * scale : -INFINITY;
     }
     __syncthreads();
-    for (int hq = wave; hq < nh; hq += 4) {      // the tile's maximum per head, a wave per head
-      float m = fmaxf(fmaxf(wt[hq * kTile + lane], wt[hq * kTile + 64 + lane]),
-                      fmaxf(wt[hq * kTile + 128 + lane], wt[hq * kTile + 192 + lane]));
+    for (int hq = wave; hq < nh; hq += nw) {     // the tile's maximum per head, a wave per head
+      float m = wt[hq * nthr + lane];
+      for (int u = 1; u < nw; ++u) m = fmaxf(m, wt[hq * nthr + 64 * u + lane]);
       m = wave_max(m);
       if (lane == 0) {
         const float m_old = m_run[hq], m_new = fmaxf(m_old, m);
@@ -259,13 +265,13 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
 #pragma unroll
     for (int hq = 0; hq < NH; ++hq)
       if (hq < nh) {
-        const float sv = wt[hq * kTile + tid];
-        wt[hq * kTile + tid] = idx < total ? expf(sv - m_run[hq]) : 0.f;
+        const float sv = wt[hq * nthr + tid];
+        wt[hq * nthr + tid] = idx < key_hi ? expf(sv - m_run[hq]) : 0.f;
       }
     __syncthreads();
-    for (int hq = wave; hq < nh; hq += 4) {      // running sum of the weights
-      float sum = (wt[hq * kTile + lane] + wt[hq * kTile + 64 + lane]) +
-                  (wt[hq * kTile + 128 + lane] + wt[hq * kTile + 192 + lane]);
+    for (int hq = wave; hq < nh; hq += nw) {     // running sum of the weights
+      float sum = wt[hq * nthr + lane];
+      for (int u = 1; u < nw; ++u) sum += wt[hq * nthr + 64 * u + lane];
       sum = wave_sum(sum);
       if (lane == 0) l_run[hq] = l_run[hq] * corr[hq] + sum;
     }
@@ -276,13 +282,13 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
 #pragma unroll
         for (int m = 0; m < NC; ++m) acc[hq][m] *= cf;
       }
-    const int n_here = total - base < kTile ? total - base : kTile;
-    constexpr int kBatch = NC <= 2 ? 16 : (NC <= 4 ? 8 : 4);   // value rows a wave has in flight
-    for (int kk0 = wave; kk0 < n_here; kk0 += 4 * kBatch) {
+    const int n_here = key_hi - base < nthr ? key_hi - base : nthr;
+    constexpr int kBatch = NC <= 2 ? 16 : (NC <= 4 || NH <= 4 ? 8 : 4);   // value rows a wave has in flight
+    for (int kk0 = wave; kk0 < n_here; kk0 += nw * kBatch) {
       float vf[kBatch][NC];
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        const int kk = kk0 + 4 * u < n_here ? kk0 + 4 * u : n_here - 1;
+        const int kk = kk0 + nw * u < n_here ? kk0 + nw * u : n_here - 1;
         const size_t at = vat[kk];
 #pragma unroll
         for (int m = 0; m < NC; ++m)
@@ -290,12 +296,12 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       }
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        const int kk = kk0 + 4 * u;
+        const int kk = kk0 + nw * u;
         if (kk < n_here) {
 #pragma unroll
           for (int hq = 0; hq < NH; ++hq)
             if (hq < nh) {
-              const float w = wt[hq * kTile + kk];
+              const float w = wt[hq * nthr + kk];
 #pragma unroll
               for (int m = 0; m < NC; ++m) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
             }
@@ -304,7 +310,8 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
     }
     __syncthreads();
   }
-  // the four waves' sums in wave order, one head at a time
+  // the waves' sums in wave order, one head at a time
+  const int R = gridDim.x;
 #pragma unroll
   for (int hq = 0; hq < NH; ++hq) {
     if (hq < nh) {
@@ -312,32 +319,80 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       for (int m = 0; m < NC; ++m)
         if (lane + 64 * m < dv) red[wave * dv + lane + 64 * m] = acc[hq][m];
       __syncthreads();
-      const float inv = 1.f / l_run[hq];
-      for (int c = tid; c < dv; c += 256) {
-        const float o = (((red[c] + red[dv + c]) + red[2 * dv + c]) + red[3 * dv + c]) * inv;
-        const size_t at = (size_t)r * H * dv + (size_t)(h0 + hq) * dv + c;
-        out[at] = o;
-        if (out_b) out_b[at] = (bf16_t)o;
+      const float inv = n_splits > 1 ? 1.f : 1.f / l_run[hq];
+      for (int c = tid; c < dv; c += nthr) {
+        float o = red[c];
+        for (int u = 1; u < nw; ++u) o += red[u * dv + c];
+        o *= inv;
+        if (n_splits > 1) {
+          part_acc[(((size_t)split * R + r) * H + h0 + hq) * dv + c] = o;
+        } else {
+          const size_t at = (size_t)r * H * dv + (size_t)(h0 + hq) * dv + c;
+          out[at] = o;
+          if (out_b) out_b[at] = (bf16_t)o;
+        }
+      }
+      if (n_splits > 1 && tid == 0) {
+        float* ml = part_ml + (((size_t)split * R + r) * H + h0 + hq) * 2;
+        ml[0] = m_run[hq];
+        ml[1] = l_run[hq];
       }
       __syncthreads();
     }
   }
 }
 
+// out[r, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), tiles s in order, M = max m_s.
+__global__ void softmax_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                     int n_splits, float* __restrict__ out, bf16_t* __restrict__ out_b, int H, int dv) {
+  const int r = blockIdx.x, h = blockIdx.y, R = gridDim.x;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(((size_t)s * R + r) * H + h) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float* ml = part_ml + (((size_t)s * R + r) * H + h) * 2;
+    if (ml[0] != -INFINITY) L += ml[1] * expf(ml[0] - M);
+  }
+  for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float m = part_ml[(((size_t)s * R + r) * H + h) * 2];
+      if (m != -INFINITY) o = fmaf(part_acc[(((size_t)s * R + r) * H + h) * dv + c], expf(m - M), o);
+    }
+    o /= L;
+    const size_t at = ((size_t)r * H + h) * dv + c;
+    out[at] = o;
+    if (out_b) out_b[at] = (bf16_t)o;
+  }
+}
+
+constexpr int kSplitRows = 64;   // batches of at most this many rows cut their keys over workgroups
+constexpr int kSplitKeys = 64;   // ... in tiles of this many keys (one wave each)
+
 template <typename T, int NH>
-void launch_softmax_nc(dim3 grid, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq, const void* kc,
-                       const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot, const int32_t* bt,
-                       int max_blocks, int page, int H, int G, int dk, int dv, int window, int keep_first, float scale,
-                       float* out, bf16_t* out_b, int n_hgroups) {
-#define SD_GO(NC)                                                                                                  \
-  window_softmax_attn_kernel<T, NH, NC><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
-                                                                row_slot, bt, max_blocks, page, H, G, dk, dv, window, \
-                                                                keep_first, scale, out, out_b, n_hgroups)
+void launch_softmax_nc(dim3 grid, int nthr, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq,
+                       const void* kc, const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot,
+                       const int32_t* bt, int max_blocks, int page, int H, int G, int dk, int dv, int window,
+                       int keep_first, float scale, float* out, bf16_t* out_b, int n_hgroups, int n_splits,
+                       float* part_acc, float* part_ml) {
+#define SD_GO2(NC, NT)                                                                                              \
+  window_softmax_attn_kernel<T, NH, NC, NT><<<grid, NT, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
+                                                                   row_slot, bt, max_blocks, page, H, G, dk, dv,       \
+                                                                   window, keep_first, scale, out, out_b, n_hgroups,   \
+                                                                   n_splits, part_acc, part_ml)
+#define SD_GO(NC)                                          \
+  do {                                                     \
+    if constexpr (NH <= 4) {                               \
+      if (nthr == kSplitKeys) { SD_GO2(NC, kSplitKeys); break; } \
+    }                                                      \
+    SD_GO2(NC, 256);                                       \
+  } while (0)
   if (nc == 1) SD_GO(1);
   else if (nc == 2) SD_GO(2);
   else if (nc == 4) SD_GO(4);
   else SD_GO(8);
 #undef SD_GO
+#undef SD_GO2
 }
 
 // ------------------------------------------------------------------ causal convolution
@@ -564,7 +619,78 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int64_t ld, i
     for (int j = 0; j < top; ++j) sel_w[(size_t)r * top + j] /= total;
 }
 
+// The router's product and the choice in one launch: a workgroup per row, a wave per expert
+// (lanes stride over the row's channels, then a butterfly sum: an order that no other row
+// changes), then the first wave chooses as moe_route_kernel does.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_rows_kernel(const float* __restrict__ x, int64_t ldx,
+                                                             const T* __restrict__ w, float* __restrict__ logits,
+                                                             int32_t* __restrict__ sel_e, float* __restrict__ sel_w,
+                                                             int E, int K, int top, int score_kind, int renorm,
+                                                             int round) {
+  extern __shared__ float sc[];   // [E]
+  const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float* xr = x + (size_t)r * ldx;
+  for (int e = wave; e < E; e += 4) {
+    const T* wr = w + (size_t)e * K;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) acc = fmaf(maybe_round(xr[k], round), ld_f(wr + k), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      sc[e] = acc;
+      if (logits) logits[(size_t)r * E + e] = acc;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  if (score_kind == 0) {
+    for (int e = lane; e < E; e += 64) sc[e] = sigmoid_f(sc[e]);
+  } else {
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, sc[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float p = expf(sc[e] - m);
+      sc[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) sc[e] /= sum;
+  }
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = sc[e];
+      if (v > best) {
+        best = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+      }
+    }
+    if (lane == 0) {
+      sel_e[(size_t)r * top + j] = bi;
+      sel_w[(size_t)r * top + j] = best;
+      sc[bi] = -INFINITY;
+    }
+    total += best;
+  }
+  if (renorm && lane == 0)
+    for (int j = 0; j < top; ++j) sel_w[(size_t)r * top + j] /= total;
+}
+
 constexpr int kMoeBM = 32;   // assignment rows per tile of the grouped products
+constexpr int kMoeDirect = 16;  // at most this many assignments: each is its own tile, nothing is grouped
 // cnt[e] = assignments of expert e.  One workgroup per expert.
 __global__ void moe_count_kernel(const int32_t* __restrict__ sel_e, int n, int32_t* __restrict__ cnt) {
   __shared__ float red[4];
@@ -620,17 +746,19 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const T* __restrict__ Wgu,
     float* __restrict__ act, int top, int F, int K, int scale_input, int round) {
   constexpr int BM = kMoeBM, BN = 64, BK = 16, TM = 2, TN = 4;
-  if ((int)blockIdx.y >= n_tiles[0]) return;
+  if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
   __shared__ float xs[BK][BM + 1];
   __shared__ float wg[BK][BN + 1];
   __shared__ float wu[BK][BN + 1];
   __shared__ int arow[BM];
-  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
+  const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
+  const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, tx = tid % (BN / TN), ty = tid / (BN / TN);
   const int n0 = blockIdx.x * BN;
   const T* Wg = Wgu + (size_t)e * 2 * F * K;
   const T* Wu = Wg + (size_t)F * K;
-  if (tid < BM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   __syncthreads();
   float ag[TM][TN], au[TM][TN];
 #pragma unroll
@@ -690,15 +818,17 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const T* __restrict__ Wd,
     float* __restrict__ out, int N, int K, int scale_input) {
   constexpr int BM = kMoeBM, BN = 64, BK = 16, TM = 2, TN = 4;
-  if ((int)blockIdx.y >= n_tiles[0]) return;
+  if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
   __shared__ float xs[BK][BM + 1];
   __shared__ float ws[BK][BN + 1];
   __shared__ int arow[BM];
-  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
+  const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
+  const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, tx = tid % (BN / TN), ty = tid / (BN / TN);
   const int n0 = blockIdx.x * BN;
   const T* W = Wd + (size_t)e * N * K;
-  if (tid < BM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   __syncthreads();
   float acc[TM][TN];
 #pragma unroll
@@ -760,16 +890,18 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
     const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wgu,
     bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
-  if ((int)blockIdx.y >= n_tiles[0]) return;
+  if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
   __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
   __shared__ int arow[kMoeBM];
-  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
+  const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
+  const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
   const int n = blockIdx.x * 64 + wave * 16 + lr;
   const int nc = n < F ? n : F - 1;
   const bf16_t* wg = Wgu + ((size_t)e * 2 * F + nc) * K + 8 * kq;
   const bf16_t* wu = wg + (size_t)F * K;
-  if (tid < kMoeBM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  if (tid < kMoeBM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   f32x4 ag[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, au[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
     const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
@@ -785,7 +917,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
       *reinterpret_cast<bf16x4*>(xs + m * kMfLd + k4) = v;
     }
     __syncthreads();
-#pragma unroll 4
+#pragma unroll 8
     for (int k0 = 0; k0 < kc; k0 += 32) {
       const bf16x8 fg = *reinterpret_cast<const bf16x8*>(wg + kc0 + k0);
       const bf16x8 fu = *reinterpret_cast<const bf16x8*>(wu + kc0 + k0);
@@ -814,15 +946,17 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
     const bf16_t* __restrict__ act, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wd,
     float* __restrict__ out, int N, int K, int scale_input) {
-  if ((int)blockIdx.y >= n_tiles[0]) return;
+  if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
   __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
   __shared__ int arow[kMoeBM];
-  const int e = tiles[3 * blockIdx.y], p0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+  // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
+  const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
+  const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 128 + wave * 32 + lr, n1 = n0 + 16;
   const bf16_t* w0 = Wd + ((size_t)e * N + (n0 < N ? n0 : N - 1)) * K + 8 * kq;
   const bf16_t* w1 = Wd + ((size_t)e * N + (n1 < N ? n1 : N - 1)) * K + 8 * kq;
-  if (tid < kMoeBM) arow[tid] = tid < rows ? perm[p0 + tid] : -1;
+  if (tid < kMoeBM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   f32x4 acc[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
   for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
     const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
@@ -835,7 +969,7 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
       *reinterpret_cast<bf16x8*>(xs + m * kMfLd + k8) = v;
     }
     __syncthreads();
-#pragma unroll 4
+#pragma unroll 8
     for (int k0 = 0; k0 < kc; k0 += 32) {
       const bf16x8 f0 = *reinterpret_cast<const bf16x8*>(w0 + kc0 + k0);
       const bf16x8 f1 = *reinterpret_cast<const bf16x8*>(w1 + kc0 + k0);
@@ -989,11 +1123,20 @@ extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int6
   return SD_OK;
 }
 
+extern "C" size_t sd_window_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window, int keep_first,
+                                                             int max_ctx) {
+  if (n_rows < 1 || n_rows > kSplitRows || H < 1 || dv < 1 || window < 1) return 0;
+  long long max_keys = (long long)window + (keep_first > 0 ? keep_first : 0);
+  if (max_keys > max_ctx) max_keys = max_ctx;
+  const int splits = (int)((max_keys + kSplitKeys - 1) / kSplitKeys);
+  return splits > 1 ? (size_t)splits * n_rows * H * (dv + 2) * sizeof(float) : 0;
+}
+
 extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
                                            int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
                                            const int32_t* block_tables, int max_blocks, int page, int n_rows, int H,
                                            int G, int dk, int dv, int window, int keep_first, float scale, float* out,
-                                           void* out_bf16, sd_stream_t stream) {
+                                           void* out_bf16, void* scratch, size_t scratch_bytes, sd_stream_t stream) {
   SD_REQUIRE(q && k_cache && row_pos && row_slot && block_tables && out, SD_ERR_INVALID,
              "sd_window_softmax_attention: null argument");
   SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && keep_first >= 0 && page >= 1,
@@ -1002,19 +1145,28 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
              "sd_window_softmax_attention: value size %d outside 1..512 (or above the key row it is part of)", dv);
   hipStream_t st = (hipStream_t)stream;
   const int qh = H / G;
-  const int NH = qh <= 1 ? 1 : (qh <= 2 ? 2 : (qh <= 4 ? 4 : 8));
+  const size_t need = sd_window_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, max_blocks * page);
+  const bool split = need > 0 && scratch && scratch_bytes >= need && sd_aligned16(scratch);
+  const int n_splits = split ? (int)(need / ((size_t)n_rows * H * (dv + 2) * sizeof(float))) : 1;
+  const int nthr = split ? kSplitKeys : 256;
+  // (a cut launch has many workgroups already: fewer heads each, so that a thread scores its key sooner)
+  const int cap = split ? 4 : 8;
+  const int NH = qh <= 1 ? 1 : (qh <= 2 ? 2 : (qh <= 4 || cap == 4 ? 4 : 8));
   const int n_hgroups = (qh + NH - 1) / NH;
   const int nc = dv <= 64 ? 1 : (dv <= 128 ? 2 : (dv <= 256 ? 4 : 8));
-  const size_t lds = sizeof(unsigned long long) * kTile +
-                     sizeof(float) * ((size_t)NH * kTile + (size_t)NH * dk + 3 * (size_t)NH + (size_t)4 * dv);
+  const size_t lds = sizeof(unsigned long long) * nthr +
+                     sizeof(float) * ((size_t)NH * nthr + (size_t)NH * dk + 3 * (size_t)NH + (size_t)(nthr / 64) * dv);
   SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_softmax_attention: dim %d / vdim %d need %zu bytes of LDS",
              dk, dv, lds);
   const void* vc = v_cache ? v_cache : k_cache;
   const int v_row = v_cache ? dv : dk;
-  dim3 grid(n_rows, G, n_hgroups);
-#define SD_NH(T, N)                                                                                              \
-  launch_softmax_nc<T, N>(grid, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables, max_blocks, \
-                          page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups)
+  float* part_acc = split ? (float*)scratch : nullptr;
+  float* part_ml = split ? part_acc + (size_t)n_splits * n_rows * H * dv : nullptr;
+  dim3 grid(n_rows, G, n_hgroups * n_splits);
+#define SD_NH(T, N)                                                                                                  \
+  launch_softmax_nc<T, N>(grid, nthr, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables,      \
+                          max_blocks, page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups, \
+                          n_splits, part_acc, part_ml)
 #define SD_T(T)                      \
   do {                               \
     if (NH == 1) SD_NH(T, 1);        \
@@ -1027,6 +1179,11 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
 #undef SD_T
 #undef SD_NH
   SD_CHECK_LAUNCH("sd_window_softmax_attention");
+  if (split) {
+    softmax_merge_kernel<<<dim3(n_rows, H), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), 0, st>>>(
+        part_acc, part_ml, n_splits, out, (bf16_t*)out_bf16, H, dv);
+    SD_CHECK_LAUNCH("sd_window_softmax_attention (merge)");
+  }
   return SD_OK;
 }
 
@@ -1112,6 +1269,25 @@ extern "C" int sd_moe_route(const float* logits, int64_t ld, int32_t* sel_expert
   return SD_OK;
 }
 
+extern "C" int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_router, int w_f32, float* logits,
+                                 int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
+                                 int score_kind, int renorm, sd_stream_t stream) {
+  SD_REQUIRE(x && w_router && sel_expert && sel_weight && n_rows >= 1 && E >= 1 && K >= 1 && top >= 1 && top <= E &&
+                 ldx >= K,
+             SD_ERR_INVALID, "sd_moe_route_rows: bad argument (E=%d top=%d)", E, top);
+  SD_REQUIRE(E <= 8192, SD_ERR_UNSUPPORTED, "sd_moe_route_rows: more than 8192 experts");
+  hipStream_t st = (hipStream_t)stream;
+  if (w_f32)
+    moe_route_rows_kernel<float><<<n_rows, 256, sizeof(float) * E, st>>>(x, ldx, (const float*)w_router, logits, sel_expert,
+                                                                         sel_weight, E, K, top, score_kind, renorm, 0);
+  else
+    moe_route_rows_kernel<bf16_t><<<n_rows, 256, sizeof(float) * E, st>>>(x, ldx, (const bf16_t*)w_router, logits,
+                                                                          sel_expert, sel_weight, E, K, top, score_kind,
+                                                                          renorm, 1);
+  SD_CHECK_LAUNCH("sd_moe_route_rows");
+  return SD_OK;
+}
+
 extern "C" size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W) {
   (void)W;
   if (n_rows < 1 || top < 1 || E < 1 || F < 1) return 0;
@@ -1137,12 +1313,18 @@ extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_ex
   int32_t* tiles = (int32_t*)(base + p.tiles);
   float* act = (float*)(base + p.act);
   const int n = n_rows * top;
-  moe_count_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt);
-  SD_CHECK_LAUNCH("sd_moe_experts (count)");
-  moe_group_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt, E, perm, tiles, n_tiles);
-  SD_CHECK_LAUNCH("sd_moe_experts (group)");
-  const int max_tiles = n / kMoeBM + E;
-  const int tiles_y = max_tiles < (n + 0) ? max_tiles : n;   // never more tiles than assignments
+  int tiles_y = n;
+  if (n <= kMoeDirect) {   // a few assignments: each runs as a tile of its own, straight from the router's choice
+    perm = const_cast<int32_t*>(sel_expert);
+    tiles = nullptr;
+  } else {
+    moe_count_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt);
+    SD_CHECK_LAUNCH("sd_moe_experts (count)");
+    moe_group_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt, E, perm, tiles, n_tiles);
+    SD_CHECK_LAUNCH("sd_moe_experts (group)");
+    const int max_tiles = n / kMoeBM + E;
+    tiles_y = max_tiles < n ? max_tiles : n;   // never more tiles than assignments
+  }
   if (w_f32) {
     moe_gate_up_kernel<float><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
                                                                             (const float*)w_gate_up, act, top, F, W, scale_input, 0);

@@ -1510,9 +1510,10 @@ extern "C" int sd_cache_append(const float*, int64_t, const float*, int64_t, voi
 }
 extern "C" int sd_window_softmax_attention(const float*, int64_t, const void*, const void*, int, const int32_t*,
                                            const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int,
-                                           float, float*, void*, sd_stream_t) {
+                                           float, float*, void*, void*, size_t, sd_stream_t) {
   UNSUPPORTED("sd_window_softmax_attention");
 }
+extern "C" size_t sd_window_softmax_attention_scratch_bytes(int, int, int, int, int, int) { return 0; }
 extern "C" int sd_causal_conv_rows(const float*, int64_t, const void*, const void*, int, float*, const int32_t*,
                                    const int32_t*, const int32_t*, int, float*, int64_t, int, int, int, int,
                                    sd_stream_t) { UNSUPPORTED("sd_causal_conv_rows"); }
@@ -1524,6 +1525,8 @@ extern "C" int sd_decay_scan_rows(const float*, const float*, int64_t, const flo
 extern "C" int sd_moe_route(const float*, int64_t, int32_t*, float*, int, int, int, int, int, sd_stream_t) {
   UNSUPPORTED("sd_moe_route");
 }
+extern "C" int sd_moe_route_rows(const float*, int64_t, const void*, int, float*, int32_t*, float*, int, int, int, int,
+                                 int, int, sd_stream_t) { UNSUPPORTED("sd_moe_route_rows"); }
 extern "C" size_t sd_moe_experts_scratch_bytes(int, int, int, int, int) { return 0; }
 extern "C" int sd_moe_experts(const float*, int64_t, const int32_t*, const float*, const void*, const void*, int,
                               float*, int, int, int, int, int, int, int, void*, size_t, sd_stream_t) {

@@ -1230,15 +1230,20 @@ def cache_append(k, v, k_cache, v_cache, row_pos, row_slot, block_tables, G, dk,
 
 
 def window_softmax_attention(q, k_cache, v_cache, row_pos, row_slot, block_tables, H, G, dk, dv, window,
-                             keep_first, scale) -> torch.Tensor:
+                             keep_first, scale, split=True) -> torch.Tensor:
     """q f32 [rows, H*dk]; caches [pages, G, PAGE, dk | dv]; v_cache None: values are the first dv
-    channels of the key rows.  Returns f32 [rows, H*dv]."""
+    channels of the key rows.  Returns f32 [rows, H*dv].  split=False: never cut a row's keys
+    over workgroups (few rows are cut by default)."""
     _f32(q, "q")
     out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
-    _lib.check(_lib.load().sd_window_softmax_attention(
+    lib = _lib.load()
+    n = int(lib.sd_window_softmax_attention_scratch_bytes(q.shape[0], H, dv, int(window), int(keep_first),
+                                                          block_tables.shape[1] * PAGE)) if split else 0
+    scratch = torch.empty(n, dtype=torch.uint8, device=q.device) if n else None
+    _lib.check(lib.sd_window_softmax_attention(
         _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(row_pos),
         _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0], H, G, dk, dv, int(window),
-        int(keep_first), float(scale), _p(out), None, _stream()), "sd_window_softmax_attention")
+        int(keep_first), float(scale), _p(out), None, _p(scratch), n, _stream()), "sd_window_softmax_attention")
     return out
 
 
@@ -1298,6 +1303,21 @@ def moe_route(logits, top, score="sigmoid", renorm=False):
     _lib.check(_lib.load().sd_moe_route(_p(logits), E, _p(sel_e), _p(sel_w), n, E, top,
                                         {"sigmoid": 0, "softmax": 1}[score], int(renorm), _stream()), "sd_moe_route")
     return sel_e, sel_w
+
+
+def moe_route_rows(x, w_router, top, score="sigmoid", renorm=False):
+    """The router's product and the choice in one launch: (experts int32 [rows, top], weights f32
+    [rows, top], logits f32 [rows, E])."""
+    _f32(x, "x")
+    n, K = x.shape
+    E = w_router.shape[0]
+    sel_e = torch.empty(n, top, dtype=torch.int32, device=x.device)
+    sel_w = torch.empty(n, top, dtype=torch.float32, device=x.device)
+    logits = torch.empty(n, E, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().sd_moe_route_rows(_p(x), K, _p(w_router), _wkind(w_router, "w_router"), _p(logits),
+                                             _p(sel_e), _p(sel_w), n, E, K, top, {"sigmoid": 0, "softmax": 1}[score],
+                                             int(renorm), _stream()), "sd_moe_route_rows")
+    return sel_e, sel_w, logits
 
 
 def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True) -> torch.Tensor:
