@@ -1206,9 +1206,11 @@ size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W);
 /* out[r*top + j] = down_e(act(gate_e u) * (up_e u)) for e = sel_expert[r, j], u = sel_weight *
  * x[r] (scale_input) or u = x[r] with the result multiplied by the weight (scale_input == 0);
  * act_kind 0: silu.  w_gate_up [E, 2F, W] (gate rows, then up rows), w_down [E, W, F]; x
- * [rows, W]; out [rows*top, W]: the caller adds a row's `top` results.  Rows are grouped by
- * expert on the device; nothing is read back.                                               */
-int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_expert, const float* sel_weight,
+ * [rows, W] (x_bf16, or NULL: the same rows as bf16, same row stride, for the matrix-core path);
+ * out [rows*top, W]: the caller adds a row's `top` results.  Rows are grouped by expert on the
+ * device; nothing is read back.                                               */
+int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, const int32_t* sel_expert,
+                   const float* sel_weight,
                    const void* w_gate_up, const void* w_down, int w_f32, float* out, int n_rows,
                    int top, int E, int F, int W, int scale_input, int act_kind, void* scratch,
                    size_t scratch_bytes, sd_stream_t stream);

@@ -366,7 +366,9 @@ def test_ssd_steps_and_scan(H, G, N_, P):
 @pytest.mark.parametrize("E,top,F,W,rows", [(4, 2, 24, 32, 9), (5, 3, 20, 40, 70), (1, 1, 8, 24, 3), (16, 1, 64, 48, 150),
                                             (7, 7, 10, 20, 5),
                                             # widths that are multiples of 32: bfloat16 takes the matrix-core kernels
-                                            (8, 2, 96, 64, 100), (3, 1, 32, 32, 33), (6, 3, 160, 1056, 5)])
+                                            (8, 2, 96, 64, 100), (3, 1, 32, 32, 33), (6, 3, 160, 1056, 5),
+                                            # many rows per expert: the matrix-core kernels take tiles of 128 rows
+                                            (4, 2, 64, 160, 301), (2, 1, 32, 64, 700)])
 @pytest.mark.parametrize("wdt", [torch.float32, torch.bfloat16])
 def test_routed_experts(E, top, F, W, rows, wdt):
     from vllm_omni_draft_amd import ops

@@ -251,7 +251,7 @@ SIGNATURES = {
     "sd_moe_route": (i32, [vp, i64, vp, vp, i32, i32, i32, i32, i32, vp]),
     "sd_moe_route_rows": (i32, [vp, i64, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
     "sd_moe_experts_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
-    "sd_moe_experts": (i32, [vp, i64, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_size_t, vp]),
+    "sd_moe_experts": (i32, [vp, vp, i64, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_size_t, vp]),
     "sd_postnorm_residual": (i32, [vp, vp, i32, C.c_float, vp, C.c_float, vp, i32, C.c_float, vp, i32, i32, vp]),
     "sd_scale_rows": (i32, [vp, i64, C.c_float, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),

@@ -1299,7 +1299,7 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
     float* dn = (float*)(base + w.dn);
     const int E = l.n_experts;
     SQ_TRY(sd_moe_route_rows(x, W, l.w_router, f32, rlog, sel_e, sel_w, R, E, W, l.top, 0, 0, stream));
-    SQ_TRY(sd_moe_experts(x, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, E, l.expert_ff, W, 1, 0,
+    SQ_TRY(sd_moe_experts(x, hb, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, E, l.expert_ff, W, 1, 0,
                           base + w.moe, w.moe_bytes, stream));
     SQ_TRY(sd_postnorm_residual(x, dn, l.top, 1.f, nullptr, 0.f, l.norm2_w, f32, eps, hb, R, W, stream));
   }

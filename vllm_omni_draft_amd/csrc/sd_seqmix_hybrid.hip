@@ -701,23 +701,24 @@ __global__ void moe_count_kernel(const int32_t* __restrict__ sel_e, int n, int32
   if (threadIdx.x == 0) cnt[e] = (int)c;
 }
 // perm: assignments grouped by expert, ascending inside a group; tiles[t] = {expert, first index
-// in perm, rows}; n_tiles[0] = number of tiles.  One workgroup of 256 per expert.
+// in perm, rows <= bm}; n_tiles[0] = number of tiles.  One workgroup of 256 per expert.
 __global__ void moe_group_kernel(const int32_t* __restrict__ sel_e, int n, const int32_t* __restrict__ cnt, int E,
-                                 int32_t* __restrict__ perm, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles) {
+                                 int32_t* __restrict__ perm, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles,
+                                 int bm) {
   __shared__ int wsum[4];
   __shared__ int base_s;
   const int e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   int off = 0, toff = 0;
   for (int i = 0; i < e; ++i) {
     off += cnt[i];
-    toff += (cnt[i] + kMoeBM - 1) / kMoeBM;
+    toff += (cnt[i] + bm - 1) / bm;
   }
   const int mine = cnt[e];
-  const int my_tiles = (mine + kMoeBM - 1) / kMoeBM;
+  const int my_tiles = (mine + bm - 1) / bm;
   for (int t = tid; t < my_tiles; t += 256) {
     tiles[3 * (toff + t)] = e;
-    tiles[3 * (toff + t) + 1] = off + t * kMoeBM;
-    tiles[3 * (toff + t) + 2] = mine - t * kMoeBM < kMoeBM ? mine - t * kMoeBM : kMoeBM;
+    tiles[3 * (toff + t) + 1] = off + t * bm;
+    tiles[3 * (toff + t) + 2] = mine - t * bm < bm ? mine - t * bm : bm;
   }
   if (e == E - 1 && tid == 0) n_tiles[0] = toff + my_tiles;
   if (tid == 0) base_s = 0;
@@ -874,115 +875,141 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
 }
 
 // ---- the same two products on the matrix cores (bf16 weights, K a multiple of 32).  A workgroup
-// takes one tile of kMoeBM assignment rows; its rows are staged in LDS as bf16 in chunks of
-// kMfKC columns, every wave reads its weight fragments straight from the row-major matrices
-// (a lane's 8 consecutive k of one weight row are 16 contiguous bytes).  16x16x32 tiles: operand
-// lane l holds row l%16, k-block l/16; result lane l holds rows 4*(l/16)..+3 of column l%16.
-constexpr int kMfKC = 512;
-constexpr int kMfLd = kMfKC + 8;   // LDS row stride in bf16: 16 rows at one k fall into distinct banks
-
+// takes one tile of 16*MT assignment rows; its rows are staged in LDS as bf16 in chunks of KC
+// columns, every wave reads its weight fragments straight from the row-major matrices (a lane's 8
+// consecutive k of one weight row are 16 contiguous bytes).  16x16x32 tiles: operand lane l holds
+// row l%16, k-block l/16; result lane l holds rows 4*(l/16)..+3 of column l%16.
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// act[a, n] (bf16) = silu(s * gate) * (s * up); a wave owns 16 columns of gate and of up.
+// act[a, n] (bf16) = silu(s * gate) * (s * up); a wave owns 32 columns of gate and of up.  Xb (or
+// nullptr): the rows of X as bf16 already.
+template <int MT, int KC>
 __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
-    const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
-    const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wgu,
-    bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
+    const float* __restrict__ X, const bf16_t* __restrict__ Xb, int64_t ldx, const int32_t* __restrict__ perm,
+    const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w,
+    const bf16_t* __restrict__ Wgu, bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
   if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
-  __shared__ int arow[kMoeBM];
+  constexpr int BM = 16 * MT, LD = KC + 8;   // LDS row stride: 16 rows at one k fall into distinct banks
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LD];
+  __shared__ int arow[BM];
   // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
   const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
   const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
-  const int n = blockIdx.x * 64 + wave * 16 + lr;
-  const int nc = n < F ? n : F - 1;
-  const bf16_t* wg = Wgu + ((size_t)e * 2 * F + nc) * K + 8 * kq;
-  const bf16_t* wu = wg + (size_t)F * K;
-  if (tid < kMoeBM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
-  f32x4 ag[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, au[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-  for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
-    const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
+  const int n0 = blockIdx.x * 128 + wave * 32 + lr, n1 = n0 + 16;
+  const bf16_t* wg0 = Wgu + ((size_t)e * 2 * F + (n0 < F ? n0 : F - 1)) * K + 8 * kq;
+  const bf16_t* wg1 = Wgu + ((size_t)e * 2 * F + (n1 < F ? n1 : F - 1)) * K + 8 * kq;
+  const bf16_t* wu0 = wg0 + (size_t)F * K;
+  const bf16_t* wu1 = wg1 + (size_t)F * K;
+  if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
+  f32x4 ag[MT][2], au[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) ag[mt][0] = ag[mt][1] = au[mt][0] = au[mt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int m_tiles = (rows + 15) / 16;
+  for (int kc0 = 0; kc0 < K; kc0 += KC) {
+    const int kc = K - kc0 < KC ? K - kc0 : KC;
     __syncthreads();
-    for (int idx = tid; idx < kMoeBM * (kc / 4); idx += 256) {
-      const int m = idx / (kc / 4), k4 = (idx % (kc / 4)) * 4;
-      const int a = arow[m];
-      bf16x4 v = {0, 0, 0, 0};
-      if (a >= 0) {
-        const float* xr = X + (size_t)(a / top) * ldx + kc0 + k4;
-        v = bf16x4{(bf16_t)xr[0], (bf16_t)xr[1], (bf16_t)xr[2], (bf16_t)xr[3]};
+    if (Xb) {
+      for (int idx = tid; idx < 16 * m_tiles * (kc / 8); idx += 256) {
+        const int m = idx / (kc / 8), k8 = (idx % (kc / 8)) * 8;
+        const int a = arow[m];
+        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (a >= 0) v = *reinterpret_cast<const bf16x8*>(Xb + (size_t)(a / top) * ldx + kc0 + k8);
+        *reinterpret_cast<bf16x8*>(xs + m * LD + k8) = v;
       }
-      *reinterpret_cast<bf16x4*>(xs + m * kMfLd + k4) = v;
+    } else {
+      for (int idx = tid; idx < 16 * m_tiles * (kc / 4); idx += 256) {
+        const int m = idx / (kc / 4), k4 = (idx % (kc / 4)) * 4;
+        const int a = arow[m];
+        bf16x4 v = {0, 0, 0, 0};
+        if (a >= 0) {
+          const f32x4 xv = *reinterpret_cast<const f32x4*>(X + (size_t)(a / top) * ldx + kc0 + k4);
+          v = bf16x4{(bf16_t)xv[0], (bf16_t)xv[1], (bf16_t)xv[2], (bf16_t)xv[3]};
+        }
+        *reinterpret_cast<bf16x4*>(xs + m * LD + k4) = v;
+      }
     }
     __syncthreads();
-#pragma unroll 8
+#pragma unroll(KC / 32 <= 4 ? KC / 32 : 4)
     for (int k0 = 0; k0 < kc; k0 += 32) {
-      const bf16x8 fg = *reinterpret_cast<const bf16x8*>(wg + kc0 + k0);
-      const bf16x8 fu = *reinterpret_cast<const bf16x8*>(wu + kc0 + k0);
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(xs + lr * kMfLd + k0 + 8 * kq);
-      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(xs + (16 + lr) * kMfLd + k0 + 8 * kq);
-      ag[0] = mfma16(a0, fg, ag[0]);
-      ag[1] = mfma16(a1, fg, ag[1]);
-      au[0] = mfma16(a0, fu, au[0]);
-      au[1] = mfma16(a1, fu, au[1]);
+      const bf16x8 fg0 = *reinterpret_cast<const bf16x8*>(wg0 + kc0 + k0);
+      const bf16x8 fg1 = *reinterpret_cast<const bf16x8*>(wg1 + kc0 + k0);
+      const bf16x8 fu0 = *reinterpret_cast<const bf16x8*>(wu0 + kc0 + k0);
+      const bf16x8 fu1 = *reinterpret_cast<const bf16x8*>(wu1 + kc0 + k0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt < m_tiles) {
+          const bf16x8 a = *reinterpret_cast<const bf16x8*>(xs + (16 * mt + lr) * LD + k0 + 8 * kq);
+          ag[mt][0] = mfma16(a, fg0, ag[mt][0]);
+          ag[mt][1] = mfma16(a, fg1, ag[mt][1]);
+          au[mt][0] = mfma16(a, fu0, au[mt][0]);
+          au[mt][1] = mfma16(a, fu1, au[mt][1]);
+        }
+      }
     }
   }
-  if (n >= F) return;
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int a = arow[mt * 16 + 4 * kq + i];
       if (a < 0) continue;
       const float sc = scale_input ? sel_w[a] : 1.f;
-      act[(size_t)a * F + n] = (bf16_t)(silu_f(sc * ag[mt][i]) * (sc * au[mt][i]));
+      if (n0 < F) act[(size_t)a * F + n0] = (bf16_t)(silu_f(sc * ag[mt][0][i]) * (sc * au[mt][0][i]));
+      if (n1 < F) act[(size_t)a * F + n1] = (bf16_t)(silu_f(sc * ag[mt][1][i]) * (sc * au[mt][1][i]));
     }
 }
 
 // out[a, n] = down_e act[a]; a wave owns 32 columns.
+template <int MT, int KC>
 __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
     const bf16_t* __restrict__ act, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const bf16_t* __restrict__ Wd,
     float* __restrict__ out, int N, int K, int scale_input) {
   if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[kMoeBM * kMfLd];
-  __shared__ int arow[kMoeBM];
-  // (tiles == nullptr: assignment blockIdx.y alone, perm is then the chosen experts themselves)
+  constexpr int BM = 16 * MT, LD = KC + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LD];
+  __shared__ int arow[BM];
   const int e = tiles ? tiles[3 * blockIdx.y] : perm[blockIdx.y];
   const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 128 + wave * 32 + lr, n1 = n0 + 16;
   const bf16_t* w0 = Wd + ((size_t)e * N + (n0 < N ? n0 : N - 1)) * K + 8 * kq;
   const bf16_t* w1 = Wd + ((size_t)e * N + (n1 < N ? n1 : N - 1)) * K + 8 * kq;
-  if (tid < kMoeBM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
-  f32x4 acc[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
-  for (int kc0 = 0; kc0 < K; kc0 += kMfKC) {
-    const int kc = K - kc0 < kMfKC ? K - kc0 : kMfKC;
+  if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
+  f32x4 acc[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt][0] = acc[mt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int m_tiles = (rows + 15) / 16;
+  for (int kc0 = 0; kc0 < K; kc0 += KC) {
+    const int kc = K - kc0 < KC ? K - kc0 : KC;
     __syncthreads();
-    for (int idx = tid; idx < kMoeBM * (kc / 8); idx += 256) {
+    for (int idx = tid; idx < 16 * m_tiles * (kc / 8); idx += 256) {
       const int m = idx / (kc / 8), k8 = (idx % (kc / 8)) * 8;
       const int a = arow[m];
       bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (a >= 0) v = *reinterpret_cast<const bf16x8*>(act + (size_t)a * K + kc0 + k8);
-      *reinterpret_cast<bf16x8*>(xs + m * kMfLd + k8) = v;
+      *reinterpret_cast<bf16x8*>(xs + m * LD + k8) = v;
     }
     __syncthreads();
-#pragma unroll 8
+#pragma unroll(KC / 32 <= 8 ? KC / 32 : 8)
     for (int k0 = 0; k0 < kc; k0 += 32) {
       const bf16x8 f0 = *reinterpret_cast<const bf16x8*>(w0 + kc0 + k0);
       const bf16x8 f1 = *reinterpret_cast<const bf16x8*>(w1 + kc0 + k0);
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(xs + lr * kMfLd + k0 + 8 * kq);
-      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(xs + (16 + lr) * kMfLd + k0 + 8 * kq);
-      acc[0][0] = mfma16(a0, f0, acc[0][0]);
-      acc[1][0] = mfma16(a1, f0, acc[1][0]);
-      acc[0][1] = mfma16(a0, f1, acc[0][1]);
-      acc[1][1] = mfma16(a1, f1, acc[1][1]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt < m_tiles) {
+          const bf16x8 a = *reinterpret_cast<const bf16x8*>(xs + (16 * mt + lr) * LD + k0 + 8 * kq);
+          acc[mt][0] = mfma16(a, f0, acc[mt][0]);
+          acc[mt][1] = mfma16(a, f1, acc[mt][1]);
+        }
+      }
     }
   }
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int a = arow[mt * 16 + 4 * kq + i];
@@ -1294,7 +1321,8 @@ extern "C" size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F
   return moe_plan(n_rows, top, E, F).total;
 }
 
-extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_expert, const float* sel_weight,
+extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, const int32_t* sel_expert,
+                              const float* sel_weight,
                               const void* w_gate_up, const void* w_down, int w_f32, float* out, int n_rows, int top,
                               int E, int F, int W, int scale_input, int act_kind, void* scratch, size_t scratch_bytes,
                               sd_stream_t stream) {
@@ -1313,6 +1341,11 @@ extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_ex
   int32_t* tiles = (int32_t*)(base + p.tiles);
   float* act = (float*)(base + p.act);
   const int n = n_rows * top;
+  const bool mfma = !w_f32 && W % 32 == 0 && F % 32 == 0 && sd_aligned16(w_gate_up) && sd_aligned16(w_down) &&
+                    ldx % 8 == 0 && sd_aligned16(x) && (!x_bf16 || sd_aligned16(x_bf16));
+  // (tiles of 128 rows for experts with many rows, the template's MT = 8 with chunks of 128 columns,
+  // measured slower than tiles of 32: 95-156 against 153-183 TFLOP/s at 1024-2048 rows)
+  const int bm = kMoeBM;
   int tiles_y = n;
   if (n <= kMoeDirect) {   // a few assignments: each runs as a tile of its own, straight from the router's choice
     perm = const_cast<int32_t*>(sel_expert);
@@ -1320,9 +1353,9 @@ extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_ex
   } else {
     moe_count_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt);
     SD_CHECK_LAUNCH("sd_moe_experts (count)");
-    moe_group_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt, E, perm, tiles, n_tiles);
+    moe_group_kernel<<<E, 256, 0, st>>>(sel_expert, n, cnt, E, perm, tiles, n_tiles, bm);
     SD_CHECK_LAUNCH("sd_moe_experts (group)");
-    const int max_tiles = n / kMoeBM + E;
+    const int max_tiles = n / bm + E;
     tiles_y = max_tiles < n ? max_tiles : n;   // never more tiles than assignments
   }
   if (w_f32) {
@@ -1331,15 +1364,16 @@ extern "C" int sd_moe_experts(const float* x, int64_t ldx, const int32_t* sel_ex
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_kernel<float><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
                                                                          (const float*)w_down, out, W, F, scale_input);
-  } else if (W % 32 == 0 && F % 32 == 0 && sd_aligned16(w_gate_up) && sd_aligned16(w_down)) {
+  } else if (mfma) {
     // (act holds n * F floats: its first half serves as the bf16 activations)
     bf16_t* act_b = (bf16_t*)act;
-    moe_gate_up_mfma_kernel<<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
-                                                                          (const bf16_t*)w_gate_up, act_b, top, F, W,
-                                                                          scale_input);
+    const dim3 g1((F + 127) / 128, tiles_y), g2((W + 127) / 128, tiles_y);
+    const bf16_t* xb = (const bf16_t*)x_bf16;
+    moe_gate_up_mfma_kernel<2, 512><<<g1, 256, 0, st>>>(x, xb, ldx, perm, tiles, n_tiles, sel_weight,
+                                                        (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
-    moe_down_mfma_kernel<<<dim3((W + 127) / 128, tiles_y), 256, 0, st>>>(act_b, perm, tiles, n_tiles, sel_weight,
-                                                                         (const bf16_t*)w_down, out, W, F, scale_input);
+    moe_down_mfma_kernel<2, 512><<<g2, 256, 0, st>>>(act_b, perm, tiles, n_tiles, sel_weight, (const bf16_t*)w_down,
+                                                     out, W, F, scale_input);
   } else {
     moe_gate_up_kernel<bf16_t><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
                                                                              (const bf16_t*)w_gate_up, act, top, F, W, scale_input, 1);

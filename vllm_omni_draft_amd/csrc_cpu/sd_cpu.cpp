@@ -1528,7 +1528,7 @@ extern "C" int sd_moe_route(const float*, int64_t, int32_t*, float*, int, int, i
 extern "C" int sd_moe_route_rows(const float*, int64_t, const void*, int, float*, int32_t*, float*, int, int, int, int,
                                  int, int, sd_stream_t) { UNSUPPORTED("sd_moe_route_rows"); }
 extern "C" size_t sd_moe_experts_scratch_bytes(int, int, int, int, int) { return 0; }
-extern "C" int sd_moe_experts(const float*, int64_t, const int32_t*, const float*, const void*, const void*, int,
+extern "C" int sd_moe_experts(const float*, const void*, int64_t, const int32_t*, const float*, const void*, const void*, int,
                               float*, int, int, int, int, int, int, int, void*, size_t, sd_stream_t) {
   UNSUPPORTED("sd_moe_experts");
 }

@@ -1330,7 +1330,7 @@ def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True) -> torch.T
     nb = int(lib.sd_moe_experts_scratch_bytes(n, top, E, F, W))
     scratch = torch.empty(nb, dtype=torch.uint8, device=x.device)
     out = torch.empty(n, top, W, dtype=torch.float32, device=x.device)
-    _lib.check(lib.sd_moe_experts(_p(x), W, _p(sel_e), _p(sel_w), _p(w_gate_up), _p(w_down), _wkind(w_down, "w_down"),
+    _lib.check(lib.sd_moe_experts(_p(x), None, W, _p(sel_e), _p(sel_w), _p(w_gate_up), _p(w_down), _wkind(w_down, "w_down"),
                                   _p(out), n, top, E, F, W, int(scale_input), 0, _p(scratch), nb, _stream()),
                "sd_moe_experts")
     return out
