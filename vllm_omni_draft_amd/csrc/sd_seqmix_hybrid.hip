@@ -623,18 +623,30 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int64_t ld, i
 // (lanes stride over the row's channels, then a butterfly sum: an order that no other row
 // changes), then the first wave chooses as moe_route_kernel does.
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_rows_kernel(const float* __restrict__ x, int64_t ldx,
+__global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __restrict__ x, int64_t ldx,
                                                              const T* __restrict__ w, float* __restrict__ logits,
                                                              int32_t* __restrict__ sel_e, float* __restrict__ sel_w,
                                                              int E, int K, int top, int score_kind, int renorm,
                                                              int round) {
   extern __shared__ float sc[];   // [E]
-  const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const float* xr = x + (size_t)r * ldx;
-  for (int e = wave; e < E; e += 4) {
+  constexpr int kU = 8;   // loads of a lane in flight
+  for (int e = wave; e < E; e += nw) {
     const T* wr = w + (size_t)e * K;
     float acc = 0.f;
-    for (int k = lane; k < K; k += 64) acc = fmaf(maybe_round(xr[k], round), ld_f(wr + k), acc);
+    for (int k0 = 0; k0 < K; k0 += 64 * kU) {
+      float xv[kU], wv[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {   // unguarded, on an index clamped into the row
+        const int k = k0 + 64 * u + lane < K ? k0 + 64 * u + lane : K - 1;
+        xv[u] = xr[k];
+        wv[u] = ld_f(wr + k);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (k0 + 64 * u + lane < K) acc = fmaf(maybe_round(xv[u], round), wv[u], acc);
+    }
     acc = wave_sum(acc);
     if (lane == 0) {
       sc[e] = acc;
@@ -1304,11 +1316,12 @@ extern "C" int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_rout
              SD_ERR_INVALID, "sd_moe_route_rows: bad argument (E=%d top=%d)", E, top);
   SD_REQUIRE(E <= 8192, SD_ERR_UNSUPPORTED, "sd_moe_route_rows: more than 8192 experts");
   hipStream_t st = (hipStream_t)stream;
+  const int nthr = 64 * (E >= 16 ? 16 : (E >= 8 ? 8 : 4));   // a wave per expert, up to 16 at a time
   if (w_f32)
-    moe_route_rows_kernel<float><<<n_rows, 256, sizeof(float) * E, st>>>(x, ldx, (const float*)w_router, logits, sel_expert,
-                                                                         sel_weight, E, K, top, score_kind, renorm, 0);
+    moe_route_rows_kernel<float><<<n_rows, nthr, sizeof(float) * E, st>>>(x, ldx, (const float*)w_router, logits, sel_expert,
+                                                                          sel_weight, E, K, top, score_kind, renorm, 0);
   else
-    moe_route_rows_kernel<bf16_t><<<n_rows, 256, sizeof(float) * E, st>>>(x, ldx, (const bf16_t*)w_router, logits,
+    moe_route_rows_kernel<bf16_t><<<n_rows, nthr, sizeof(float) * E, st>>>(x, ldx, (const bf16_t*)w_router, logits,
                                                                           sel_expert, sel_weight, E, K, top, score_kind,
                                                                           renorm, 1);
   SD_CHECK_LAUNCH("sd_moe_route_rows");
