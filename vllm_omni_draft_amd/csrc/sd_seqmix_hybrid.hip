@@ -148,67 +148,70 @@ template <> struct Piece<float> {
   }
 };
 
-// s[hq] += q[hq] . k, channels ascending.  vec: rows are 16-byte aligned and dk a multiple of the
-// piece size; then up to kLoads pieces are asked for before the first is used.
-template <typename KT, int NH>
-__device__ __forceinline__ void score_key(const KT* __restrict__ kr, const float* __restrict__ qs, int dk, int nh,
-                                          bool vec, float* s) {
-  constexpr int E = Piece<KT>::E;
+// s[hq] += q[hq] . k over n channels, ascending (kr and qs point at the first of them; a head's
+// query is q_stride floats from the next).  vec: rows are 16-byte aligned and n a multiple of
+// the piece size; then up to kLoads pieces are asked for before the first is used.
+template <typename KT_, int NH>
+__device__ __forceinline__ void score_key(const KT_* __restrict__ kr, const float* __restrict__ qs, int q_stride, int n,
+                                          int nh, bool vec, float* s) {
+  constexpr int E = Piece<KT_>::E;
   if (vec) {
-    for (int c = 0; c < dk; c += kLoads * E) {
+    for (int c = 0; c < n; c += kLoads * E) {
       u32x4 raw[kLoads];
 #pragma unroll
       for (int i = 0; i < kLoads; ++i) {   // unguarded, on an address clamped into the row
-        const int ci = c + i * E < dk ? c + i * E : dk - E;
+        const int ci = c + i * E < n ? c + i * E : n - E;
         raw[i] = *reinterpret_cast<const u32x4*>(kr + ci);
       }
 #pragma unroll
       for (int i = 0; i < kLoads; ++i) {
-        if (c + i * E < dk) {
+        if (c + i * E < n) {
           float kf[E];
-          Piece<KT>::unpack(raw[i], kf);
+          Piece<KT_>::unpack(raw[i], kf);
 #pragma unroll
           for (int hq = 0; hq < NH; ++hq)
             if (hq < nh) {
 #pragma unroll
-              for (int e = 0; e < E; ++e) s[hq] = fmaf(qs[hq * dk + c + i * E + e], kf[e], s[hq]);
+              for (int e = 0; e < E; ++e) s[hq] = fmaf(qs[hq * q_stride + c + i * E + e], kf[e], s[hq]);
             }
         }
       }
     }
     return;
   }
-  for (int c = 0; c < dk; ++c) {
+  for (int c = 0; c < n; ++c) {
     const float kf = ld_f(kr + c);
 #pragma unroll
     for (int hq = 0; hq < NH; ++hq)
-      if (hq < nh) s[hq] = fmaf(qs[hq * dk + c], kf, s[hq]);
+      if (hq < nh) s[hq] = fmaf(qs[hq * q_stride + c], kf, s[hq]);
   }
 }
 
-// One workgroup per (row, kv head, group of up to NH query heads of that kv head).  Per tile of
-// blockDim.x keys: a thread per key scores it against the query heads (q in LDS); the tile's
+// One workgroup of 256 threads per (row, kv head, group of up to NH query heads of that kv head).
+// Per tile of KT keys: the keys are scored against the query heads (q in LDS) by 256 / KT threads
+// each, over consecutive parts of the channels whose sums are added in part order; the tile's
 // maximum moves the running maximum and rescales what has been summed; then a wave per key, lanes
 // over value columns, adds the weighted value rows.  NC: value columns per lane (dv <= 64 * NC).
 // n_splits > 1 (few rows): workgroup (.., .., z) takes tile z / n_hgroups of the row's keys only
 // and leaves its maximum, its sum of weights and its unnormalised weighted values in part_ml /
 // part_acc; softmax_merge_kernel puts a row's tiles together in tile order.
-template <typename T, int NH, int NC, int NT>
-__global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
+template <typename T, int NH, int NC, int KT>
+__global__ __launch_bounds__(256) void window_softmax_attn_kernel(
     const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     int v_row, const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
     const int32_t* __restrict__ block_tables, int max_blocks, int page, int H, int G, int dk, int dv, int window,
     int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups, int n_splits,
     float* __restrict__ part_acc, float* __restrict__ part_ml) {
   extern __shared__ float lds[];
-  constexpr int nthr = NT, nw = NT >> 6;   // threads = keys per tile; waves
-  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [nthr] cache row of the key
-  float* wt = reinterpret_cast<float*>(vat + nthr);                      // [NH][nthr]
-  float* qs = wt + NH * nthr;                                            // [NH][dk]
+  constexpr int nthr = 256, nw = 4, PARTS = nthr / KT, KW = KT / 64;
+  unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [KT] cache row of the key
+  float* wt = reinterpret_cast<float*>(vat + KT);                        // [NH][KT]
+  float* qs = wt + NH * KT;                                              // [NH][dk]
   float* m_run = qs + NH * dk;                                           // [NH] running maximum
   float* l_run = m_run + NH;                                             // [NH] running sum
   float* corr = l_run + NH;                                              // [NH]
   float* red = corr + NH;                                                // [nw][dv]
+  float* ps = red + nw * dv;                                             // [PARTS][NH][KT] (PARTS > 1)
   const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
   const int hgroup = blockIdx.z % n_hgroups, split = blockIdx.z / n_hgroups;
   const int qh = H / G;
@@ -224,9 +227,15 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
   const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
   const int n_kept = keep_first < t_first ? keep_first : t_first;   // kept tokens that left the window
   const int total = n_kept + (i - t_first + 1);
-  const int key_lo = n_splits > 1 ? split * nthr : 0;
-  const int key_hi = n_splits > 1 ? (total < key_lo + nthr ? total : key_lo + nthr) : total;
-  const bool vec = dk % Piece<T>::E == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
+  const int key_lo = n_splits > 1 ? split * KT : 0;
+  const int key_hi = n_splits > 1 ? (total < key_lo + KT ? total : key_lo + KT) : total;
+  constexpr int E = Piece<T>::E;
+  const bool vec = dk % E == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
+  // the channels of this thread's part, in whole pieces
+  const int key = tid % KT, part = tid / KT;
+  const int unit = vec ? E : 1, units = dk / unit, per = (units + PARTS - 1) / PARTS;
+  const int c_lo = (part * per < units ? part * per : units) * unit;
+  const int c_hi = ((part + 1) * per < units ? (part + 1) * per : units) * unit;
   const int wave = tid >> 6, lane = tid & 63;
   float acc[NH][NC];
 #pragma unroll
@@ -234,8 +243,8 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
 #pragma unroll
     for (int m = 0; m < NC; ++m) acc[hq][m] = 0.f;
   __syncthreads();
-  for (int base = key_lo; base < key_hi; base += nthr) {
-    const int idx = base + tid;
+  for (int base = key_lo; base < key_hi; base += KT) {
+    const int idx = base + key;
     {
       float s[NH];
 #pragma unroll
@@ -243,17 +252,35 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
       if (idx < key_hi) {
         const int j = idx < n_kept ? idx : t_first + (idx - n_kept);
         const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
-        score_key<T, NH>(k_cache + at * dk, qs, dk, nh, vec, s);
-        vat[tid] = at;
+        if (c_hi > c_lo) score_key<T, NH>(k_cache + at * dk + c_lo, qs + c_lo, dk, c_hi - c_lo, nh, vec, s);
+        if (part == 0) vat[key] = at;
       }
+      if constexpr (PARTS == 1) {
 #pragma unroll
-      for (int hq = 0; hq < NH; ++hq)
-        if (hq < nh) wt[hq * nthr + tid] = idx < key_hi ? s[hq] * scale : -INFINITY;
+        for (int hq = 0; hq < NH; ++hq)
+          if (hq < nh) wt[hq * KT + key] = idx < key_hi ? s[hq] * scale : -INFINITY;
+      } else {
+#pragma unroll
+        for (int hq = 0; hq < NH; ++hq)
+          if (hq < nh) ps[(part * NH + hq) * KT + key] = s[hq];
+        __syncthreads();
+        if (part == 0) {
+#pragma unroll
+          for (int hq = 0; hq < NH; ++hq)
+            if (hq < nh) {
+              float sum = ps[hq * KT + key];
+#pragma unroll
+              for (int pp = 1; pp < PARTS; ++pp) sum += ps[(pp * NH + hq) * KT + key];
+              wt[hq * KT + key] = idx < key_hi ? sum * scale : -INFINITY;
+            }
+        }
+      }
     }
     __syncthreads();
     for (int hq = wave; hq < nh; hq += nw) {     // the tile's maximum per head, a wave per head
-      float m = wt[hq * nthr + lane];
-      for (int u = 1; u < nw; ++u) m = fmaxf(m, wt[hq * nthr + 64 * u + lane]);
+      float m = wt[hq * KT + lane];
+#pragma unroll
+      for (int u = 1; u < KW; ++u) m = fmaxf(m, wt[hq * KT + 64 * u + lane]);
       m = wave_max(m);
       if (lane == 0) {
         const float m_old = m_run[hq], m_new = fmaxf(m_old, m);
@@ -262,16 +289,19 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
       }
     }
     __syncthreads();
+    if (tid < KT) {
 #pragma unroll
-    for (int hq = 0; hq < NH; ++hq)
-      if (hq < nh) {
-        const float sv = wt[hq * nthr + tid];
-        wt[hq * nthr + tid] = idx < key_hi ? expf(sv - m_run[hq]) : 0.f;
-      }
+      for (int hq = 0; hq < NH; ++hq)
+        if (hq < nh) {
+          const float sv = wt[hq * KT + tid];
+          wt[hq * KT + tid] = base + tid < key_hi ? expf(sv - m_run[hq]) : 0.f;
+        }
+    }
     __syncthreads();
     for (int hq = wave; hq < nh; hq += nw) {     // running sum of the weights
-      float sum = wt[hq * nthr + lane];
-      for (int u = 1; u < nw; ++u) sum += wt[hq * nthr + 64 * u + lane];
+      float sum = wt[hq * KT + lane];
+#pragma unroll
+      for (int u = 1; u < KW; ++u) sum += wt[hq * KT + 64 * u + lane];
       sum = wave_sum(sum);
       if (lane == 0) l_run[hq] = l_run[hq] * corr[hq] + sum;
     }
@@ -282,7 +312,7 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
 #pragma unroll
         for (int m = 0; m < NC; ++m) acc[hq][m] *= cf;
       }
-    const int n_here = key_hi - base < nthr ? key_hi - base : nthr;
+    const int n_here = key_hi - base < KT ? key_hi - base : KT;
     constexpr int kBatch = NC <= 2 ? 16 : (NC <= 4 || NH <= 4 ? 8 : 4);   // value rows a wave has in flight
     for (int kk0 = wave; kk0 < n_here; kk0 += nw * kBatch) {
       float vf[kBatch][NC];
@@ -301,7 +331,7 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
 #pragma unroll
           for (int hq = 0; hq < NH; ++hq)
             if (hq < nh) {
-              const float w = wt[hq * nthr + kk];
+              const float w = wt[hq * KT + kk];
 #pragma unroll
               for (int m = 0; m < NC; ++m) acc[hq][m] = fmaf(w, vf[u][m], acc[hq][m]);
             }
@@ -322,6 +352,7 @@ __global__ __launch_bounds__(NT) void window_softmax_attn_kernel(
       const float inv = n_splits > 1 ? 1.f : 1.f / l_run[hq];
       for (int c = tid; c < dv; c += nthr) {
         float o = red[c];
+#pragma unroll
         for (int u = 1; u < nw; ++u) o += red[u * dv + c];
         o *= inv;
         if (n_splits > 1) {
@@ -367,23 +398,23 @@ __global__ void softmax_merge_kernel(const float* __restrict__ part_acc, const f
 }
 
 constexpr int kSplitRows = 64;   // batches of at most this many rows cut their keys over workgroups
-constexpr int kSplitKeys = 64;   // ... in tiles of this many keys (one wave each)
+constexpr int kSplitKeys = 64;   // ... in tiles of this many keys (four threads score a key)
 
 template <typename T, int NH>
-void launch_softmax_nc(dim3 grid, int nthr, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq,
+void launch_softmax_nc(dim3 grid, int kt, size_t lds, hipStream_t st, int nc, const float* q, int64_t ldq,
                        const void* kc, const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot,
                        const int32_t* bt, int max_blocks, int page, int H, int G, int dk, int dv, int window,
                        int keep_first, float scale, float* out, bf16_t* out_b, int n_hgroups, int n_splits,
                        float* part_acc, float* part_ml) {
-#define SD_GO2(NC, NT)                                                                                              \
-  window_softmax_attn_kernel<T, NH, NC, NT><<<grid, NT, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
-                                                                   row_slot, bt, max_blocks, page, H, G, dk, dv,       \
-                                                                   window, keep_first, scale, out, out_b, n_hgroups,   \
-                                                                   n_splits, part_acc, part_ml)
+#define SD_GO2(NC, KT)                                                                                               \
+  window_softmax_attn_kernel<T, NH, NC, KT><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
+                                                                    row_slot, bt, max_blocks, page, H, G, dk, dv,       \
+                                                                    window, keep_first, scale, out, out_b, n_hgroups,   \
+                                                                    n_splits, part_acc, part_ml)
 #define SD_GO(NC)                                          \
   do {                                                     \
     if constexpr (NH <= 4) {                               \
-      if (nthr == kSplitKeys) { SD_GO2(NC, kSplitKeys); break; } \
+      if (kt == kSplitKeys) { SD_GO2(NC, kSplitKeys); break; } \
     }                                                      \
     SD_GO2(NC, 256);                                       \
   } while (0)
@@ -1187,14 +1218,15 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
   const size_t need = sd_window_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, max_blocks * page);
   const bool split = need > 0 && scratch && scratch_bytes >= need && sd_aligned16(scratch);
   const int n_splits = split ? (int)(need / ((size_t)n_rows * H * (dv + 2) * sizeof(float))) : 1;
-  const int nthr = split ? kSplitKeys : 256;
+  const int kt = split ? kSplitKeys : 256;   // keys per tile
   // (a cut launch has many workgroups already: fewer heads each, so that a thread scores its key sooner)
   const int cap = split ? 4 : 8;
   const int NH = qh <= 1 ? 1 : (qh <= 2 ? 2 : (qh <= 4 || cap == 4 ? 4 : 8));
   const int n_hgroups = (qh + NH - 1) / NH;
   const int nc = dv <= 64 ? 1 : (dv <= 128 ? 2 : (dv <= 256 ? 4 : 8));
-  const size_t lds = sizeof(unsigned long long) * nthr +
-                     sizeof(float) * ((size_t)NH * nthr + (size_t)NH * dk + 3 * (size_t)NH + (size_t)(nthr / 64) * dv);
+  const size_t lds = sizeof(unsigned long long) * kt +
+                     sizeof(float) * ((size_t)NH * kt + (size_t)NH * dk + 3 * (size_t)NH + (size_t)4 * dv +
+                                      (kt < 256 ? (size_t)(256 / kt) * NH * kt : 0));
   SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_softmax_attention: dim %d / vdim %d need %zu bytes of LDS",
              dk, dv, lds);
   const void* vc = v_cache ? v_cache : k_cache;
@@ -1203,7 +1235,7 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
   float* part_ml = split ? part_acc + (size_t)n_splits * n_rows * H * dv : nullptr;
   dim3 grid(n_rows, G, n_hgroups * n_splits);
 #define SD_NH(T, N)                                                                                                  \
-  launch_softmax_nc<T, N>(grid, nthr, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables,      \
+  launch_softmax_nc<T, N>(grid, kt, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables,      \
                           max_blocks, page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups, \
                           n_splits, part_acc, part_ml)
 #define SD_T(T)                      \
