@@ -1147,6 +1147,26 @@ int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, vo
                     void* v_cache, int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
                     const int32_t* block_tables, int max_blocks, int page, int n_rows, int G,
                     int dk, int dv, sd_stream_t stream);
+/* Latent attention's preparation in one launch, per row: q_latent [rows, q_rank] (row stride
+ * ld) RMS-normed in place times q_norm_w (+ q_bf16, row stride ld_q_bf16, or NULL); kv [rows,
+ * kv_rank + rot_dim] (row stride ld): the first kv_rank channels normed in place times
+ * kv_norm_w, the next rot_dims channels turned as sd_rope_rows does, and the whole row appended
+ * to k_cache (one row of kv_rank + rot_dim elements per token: key and value at once).  The
+ * same values as sd_rmsnorm_parts + sd_rope_rows + sd_cache_append give.                     */
+int sd_latent_prep(float* q_latent, int q_rank, const void* q_norm_w, void* q_bf16,
+                   int64_t ld_q_bf16, float* kv, int kv_rank, int rot_dim, const void* kv_norm_w,
+                   int64_t ld, int w_f32, float eps, int rot_dims, int rot_layout,
+                   const double* inv_freq, float mag, void* k_cache, const int32_t* row_pos,
+                   const int32_t* row_slot, const int32_t* block_tables, int max_blocks, int page,
+                   int n_rows, sd_stream_t stream);
+/* q [rows, n_q] and k [rows, G*dk] (row stride ld) each RMS-normed over ALL their columns at
+ * once, in place, times q_norm_w / k_norm_w; then k and v [rows, G*dv] appended to the caches
+ * as sd_cache_append does.  One launch.                                                     */
+int sd_qk_norm_append(float* q, int n_q, const void* q_norm_w, float* k, int G, int dk,
+                      const void* k_norm_w, const float* v, int dv, int64_t ld, int w_f32, float eps,
+                      void* k_cache, void* v_cache, const int32_t* row_pos, const int32_t* row_slot,
+                      const int32_t* block_tables, int max_blocks, int page, int n_rows,
+                      sd_stream_t stream);
 /* Softmax attention over the cache sd_cache_append fills.  The row at position i sees j <= i
  * with i - j < window or j < keep_first; out[r, h] = sum_j softmax_j(q.k_j * scale) v_j, query
  * head h reads kv head h / (H/G).  v_cache == NULL: a value row is the first dv channels of its

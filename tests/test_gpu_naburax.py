@@ -292,6 +292,44 @@ def test_window_softmax_attention_many_keys(cdt):
     assert rel(one[0], out2[37]) < 2e-6
 
 
+@pytest.mark.parametrize("cdt", [torch.float32, torch.bfloat16])
+def test_fused_preparation_equals_its_pieces(cdt):
+    """The one-launch preparations of both attention kinds give the values of norm, rotation and
+    append run one after the other, in the residual buffers and in the cache."""
+    from vllm_omni_draft_amd import config, ops
+    g = torch.Generator().manual_seed(5)
+    n, qr, rk, dr, dims = 21, 20, 24, 10, 6
+    pos, slot = i32(list(range(40, 40 + n))), i32([1] * n)
+    bt = torch.zeros(2, 4, dtype=torch.int32, device=DEV)
+    bt[1] = i32([3, 0, 2, 1])
+    ql, kv = torch.randn(n, qr, generator=g), torch.randn(n, rk + dr, generator=g)
+    qw, kw = torch.randn(qr, generator=g).to(cdt), torch.randn(rk, generator=g).to(cdt)
+    f, mag = config.rotary_frequencies(dims, 1e4, {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.0})
+    rnd = cdt == torch.bfloat16
+    # pieces
+    q1 = ops.rmsnorm_parts(dev(ql), dev(qw), 1e-5, round_bf16=rnd)
+    kv1 = dev(kv)
+    kv1[:, :rk] = ops.rmsnorm_parts(dev(kv[:, :rk]), dev(kw), 1e-5, round_bf16=rnd)
+    ops.rope_rows(kv1, pos, 1, 0, rk, dims, dev(f), mag)
+    c1 = torch.zeros(4, 1, PAGE, rk + dr, dtype=cdt, device=DEV)
+    ops.cache_append(kv1, None, c1, None, pos, slot, bt, 1, rk + dr, 0)
+    # one launch
+    q2, kv2, c2 = dev(ql), dev(kv), torch.zeros_like(c1)
+    ops.latent_prep(q2, dev(qw), kv2, dev(kw), rk, dr, 1e-5, dims, dev(f), mag, c2, pos, slot, bt)
+    assert torch.equal(q1, q2) and torch.equal(kv1, kv2) and torch.equal(c1, c2)
+    # q and k normed over the whole projection, k and v appended
+    H, G, dk, dv = 6, 3, 12, 20
+    q, k, v = torch.randn(n, H * dk, generator=g), torch.randn(n, G * dk, generator=g), torch.randn(n, G * dv, generator=g)
+    qnw, knw = torch.randn(H * dk, generator=g).to(cdt), torch.randn(G * dk, generator=g).to(cdt)
+    qa, ka = ops.rmsnorm_parts(dev(q), dev(qnw), 1e-5), ops.rmsnorm_parts(dev(k), dev(knw), 1e-5)
+    kc1, vc1 = torch.zeros(4, G, PAGE, dk, dtype=cdt, device=DEV), torch.zeros(4, G, PAGE, dv, dtype=cdt, device=DEV)
+    ops.cache_append(ka, dev(v), kc1, vc1, pos, slot, bt, G, dk, dv)
+    qb, kb, kc2, vc2 = dev(q), dev(k), torch.zeros_like(kc1), torch.zeros_like(vc1)
+    ops.qk_norm_append(qb, dev(qnw), kb, dev(knw), dev(v), G, dk, dv, 1e-5, kc2, vc2, pos, slot, bt)
+    assert torch.equal(qa, qb) and torch.equal(ka, kb) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    assert rel(qb, N.rms_norm(q.double(), qnw.double(), 1e-5)) < 1e-6
+
+
 @pytest.mark.parametrize("M,B,N_,K", [(1, 3, 7, 5), (5, 2, 130, 24), (40, 6, 16, 136)])
 @pytest.mark.parametrize("wdt", [torch.float32, torch.bfloat16])
 def test_matmul_rows_batched(M, B, N_, K, wdt):

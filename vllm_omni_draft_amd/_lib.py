@@ -240,6 +240,10 @@ SIGNATURES = {
     "sd_rmsnorm_parts": (i32, [vp, i64, vp, i64, vp, i32, C.c_float, vp, i64, vp, i64, i32, i32, i32, i32, vp]),
     "sd_rope_rows": (i32, [vp, i64, vp, i32, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
     "sd_rope_copy_rows": (i32, [vp, i64, i32, i32, vp, i64, i32, i32, vp, i32, i32, i32, i32, i32, vp, C.c_float, vp]),
+    "sd_latent_prep": (i32, [vp, i32, vp, vp, i64, vp, i32, i32, vp, i64, i32, C.c_float, i32, i32, vp, C.c_float, vp,
+                             vp, vp, vp, i32, i32, i32, vp]),
+    "sd_qk_norm_append": (i32, [vp, i32, vp, vp, i32, i32, vp, vp, i32, i64, i32, C.c_float, vp, vp, vp, vp, vp, i32,
+                                i32, i32, vp]),
     "sd_cache_append": (i32, [vp, i64, vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
     "sd_window_softmax_attention_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32, i32]),
     "sd_window_softmax_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32,

@@ -1234,17 +1234,12 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
     float* pq = (float*)(base + w.pq);
     float* qe = (float*)(base + w.qe);
     bf16_t* cqb = (bf16_t*)(base + w.cqb);
-    // queries: latent, norm, expansion; the rotated part of each head turned
-    SQ_TRY(sd_rmsnorm_parts(proj + c.dq, ld, nullptr, 0, l.dq_norm_w, f32, eps, proj + c.dq, ld,
-                            l.w_uq_tiled ? cqb : nullptr, qr, R, qr, 1, rnd, stream));
+    // both latents normed, the shared rotated key part turned, the row [latent | rotated part] cached: one launch
+    SQ_TRY(sd_latent_prep(proj + c.dq, qr, l.dq_norm_w, l.w_uq_tiled ? cqb : nullptr, qr, proj + c.dkv, rk, dr,
+                          l.dkv_norm_w, ld, f32, eps, l.rot_dims, 1, l.inv_freq, l.rot_mag, l.k_cache, b.row_pos,
+                          b.row_slot, b.block_tables, b.max_blocks, b.page, R, stream));
     SQ_TRY(seq_linear(l.w_uq, l.w_uq_tiled, f32, proj + c.dq, nullptr, ld, cqb, qr, nullptr, pq, (int64_t)H * dh, R,
                       H * dh, qr, wide_ws, w.wide_bytes, stream));
-    // the cached row: normed latent, then the shared rotated key part
-    SQ_TRY(sd_rmsnorm_parts(proj + c.dkv, ld, nullptr, 0, l.dkv_norm_w, f32, eps, proj + c.dkv, ld, nullptr, 0, R, rk,
-                            1, rnd, stream));
-    SQ_TRY(sd_rope_rows(proj + c.dkv + rk, ld, b.row_pos, R, 1, 0, 0, l.rot_dims, 1, l.inv_freq, l.rot_mag, stream));
-    SQ_TRY(sd_cache_append(proj + c.dkv, ld, nullptr, 0, l.k_cache, nullptr, f32, b.row_pos, b.row_slot,
-                           b.block_tables, b.max_blocks, b.page, R, 1, de, 0, stream));
     // a head's query against the latent: its key expansion, transposed, applied to the unrotated
     // part; the rotated part is turned into place behind it
     SQ_TRY(sd_matmul_rows_batched(pq, (int64_t)H * dh, dh, l.w_uk_t, f32, (int64_t)rk * dk, qe, (int64_t)H * de, de,
@@ -1264,12 +1259,9 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
   } else {
     const int G = l.kv_heads;
     // attention: q and k normed over the whole projection, no rotation
-    SQ_TRY(sd_rmsnorm_parts(proj + c.q, ld, nullptr, 0, l.q_norm_w, f32, eps, proj + c.q, ld, nullptr, 0, R, H * dk, 1,
-                            0, stream));
-    SQ_TRY(sd_rmsnorm_parts(proj + c.k, ld, nullptr, 0, l.k_norm_w, f32, eps, proj + c.k, ld, nullptr, 0, R, G * dk, 1,
-                            0, stream));
-    SQ_TRY(sd_cache_append(proj + c.k, ld, proj + c.v, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
-                           b.block_tables, b.max_blocks, b.page, R, G, dk, dv, stream));
+    SQ_TRY(sd_qk_norm_append(proj + c.q, H * dk, l.q_norm_w, proj + c.k, G, dk, l.k_norm_w, proj + c.v, dv, ld, f32, eps,
+                             l.k_cache, l.v_cache, b.row_pos, b.row_slot, b.block_tables, b.max_blocks, b.page, R,
+                             stream));
     SQ_TRY(sd_window_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
                                        b.block_tables, b.max_blocks, b.page, R, H, G, dk, dv, l.window, l.keep_first,
                                        l.score_scale, o, l.w_o_tiled ? yb : nullptr, base + w.attn, w.attn_bytes,

@@ -426,6 +426,89 @@ void launch_softmax_nc(dim3 grid, int kt, size_t lds, hipStream_t st, int nc, co
 #undef SD_GO2
 }
 
+// ------------------------------------------------------------------ fused preparation of attention inputs
+// Row norm over n columns in place (times w, rounded to bf16 values when round), by a whole
+// workgroup of 256 threads: the sums of rmsnorm_parts_kernel with one part, the same bits.
+template <typename T>
+__device__ __forceinline__ void norm_in_place(float* __restrict__ v, const T* __restrict__ w, int n, float eps,
+                                              int round, bf16_t* __restrict__ copy, float* red) {
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) ss = fmaf(v[c], v[c], ss);
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)n + eps);
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const float o = maybe_round(v[c] * rstd * ld_f(w + c), round);
+    v[c] = o;
+    if (copy) copy[c] = (bf16_t)o;
+  }
+}
+
+// Latent attention, per row.  Workgroup (r, 0): the query latent normed in place (+ bf16 copy).
+// Workgroup (r, 1): the key/value latent normed in place, the shared rotated part turned in place,
+// and the row [latent | rotated part] appended to the cache.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(
+    float* __restrict__ q_lat, int q_rank, const T* __restrict__ q_w, bf16_t* __restrict__ q_copy, int64_t ld_copy,
+    float* __restrict__ kv, int kv_rank, int rot_dim, const T* __restrict__ kv_w, int64_t ld, float eps, int round,
+    int dims, int layout, const double* __restrict__ inv_freq, float mag, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_slot, const int32_t* __restrict__ block_tables, int max_blocks, int page,
+    T* __restrict__ k_cache) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  if (blockIdx.y == 0) {
+    norm_in_place<T>(q_lat + (size_t)r * ld, q_w, q_rank, eps, round, q_copy ? q_copy + (size_t)r * ld_copy : nullptr, red);
+    return;
+  }
+  float* row = kv + (size_t)r * ld;
+  norm_in_place<T>(row, kv_w, kv_rank, eps, round, nullptr, red);
+  const int pos = row_pos[r];
+  float* vec = row + kv_rank;
+  for (int i = threadIdx.x; i < dims / 2; i += blockDim.x) {
+    const double a = (double)pos * inv_freq[i];
+    const float cs = (float)cos(a) * mag, sn = (float)sin(a) * mag;
+    const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
+    const float u = vec[iu], v = vec[iv];
+    vec[iu] = u * cs - v * sn;
+    vec[iv] = v * cs + u * sn;
+  }
+  __syncthreads();
+  const int de = kv_rank + rot_dim;
+  const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+  T* dst = k_cache + ((size_t)pg * page + pos % page) * de;
+  for (int c = threadIdx.x; c < de; c += blockDim.x) st_f(dst + c, row[c]);
+}
+
+// Attention whose q and k are normed over the whole projection, per row.  Workgroup (r, 0): q
+// normed in place.  Workgroup (r, 1): k normed in place, then the key and value rows appended.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_append_kernel(
+    float* __restrict__ q, int nq, const T* __restrict__ q_w, float* __restrict__ k, int G, int dk,
+    const T* __restrict__ k_w, const float* __restrict__ v, int dv, int64_t ld, float eps,
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+    const int32_t* __restrict__ block_tables, int max_blocks, int page, T* __restrict__ k_cache,
+    T* __restrict__ v_cache) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  if (blockIdx.y == 0) {
+    norm_in_place<T>(q + (size_t)r * ld, q_w, nq, eps, 0, nullptr, red);
+    return;
+  }
+  float* kr = k + (size_t)r * ld;
+  norm_in_place<T>(kr, k_w, G * dk, eps, 0, nullptr, red);
+  __syncthreads();
+  const int pos = row_pos[r];
+  const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+  for (int c = threadIdx.x; c < G * dk; c += blockDim.x) {
+    const int g = c / dk;
+    st_f(k_cache + (((size_t)pg * G + g) * page + pos % page) * dk + c % dk, kr[c]);
+  }
+  const float* vr = v + (size_t)r * ld;
+  for (int c = threadIdx.x; c < G * dv; c += blockDim.x) {
+    const int g = c / dv;
+    st_f(v_cache + (((size_t)pg * G + g) * page + pos % page) * dv + c % dv, vr[c]);
+  }
+}
+
 // ------------------------------------------------------------------ causal convolution
 // out[r, c] = act(b[c] + sum_j w[c, taps-1-j] * in(r, j)).  One workgroup per (row, 256 channels).
 template <typename T>
@@ -1172,6 +1255,55 @@ extern "C" int sd_rope_rows(float* x, int64_t ld, const int32_t* row_pos, int n_
                             sd_stream_t stream) {
   return sd_rope_copy_rows(x, ld, head_stride, offset, x, ld, head_stride, offset, row_pos, n_rows, heads, rot_dims,
                            rot_dims, rot_layout, inv_freq, mag, stream);
+}
+
+extern "C" int sd_latent_prep(float* q_latent, int q_rank, const void* q_norm_w, void* q_bf16, int64_t ld_q_bf16,
+                              float* kv, int kv_rank, int rot_dim, const void* kv_norm_w, int64_t ld, int w_f32,
+                              float eps, int rot_dims, int rot_layout, const double* inv_freq, float mag, void* k_cache,
+                              const int32_t* row_pos, const int32_t* row_slot, const int32_t* block_tables,
+                              int max_blocks, int page, int n_rows, sd_stream_t stream) {
+  SD_REQUIRE(q_latent && q_norm_w && kv && kv_norm_w && k_cache && row_pos && row_slot && block_tables, SD_ERR_INVALID,
+             "sd_latent_prep: null argument");
+  SD_REQUIRE(n_rows >= 1 && q_rank >= 1 && kv_rank >= 1 && rot_dim >= 0 && page >= 1 && max_blocks >= 1, SD_ERR_INVALID,
+             "sd_latent_prep: bad shape");
+  SD_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim && (rot_dims == 0 || inv_freq), SD_ERR_INVALID,
+             "sd_latent_prep: rot_dims %d must be even, at most rot_dim %d, with a frequency table", rot_dims, rot_dim);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, 2);
+  if (w_f32)
+    latent_prep_kernel<float><<<grid, 256, 0, st>>>(q_latent, q_rank, (const float*)q_norm_w, (bf16_t*)q_bf16, ld_q_bf16,
+                                                    kv, kv_rank, rot_dim, (const float*)kv_norm_w, ld, eps, 0, rot_dims,
+                                                    rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
+                                                    max_blocks, page, (float*)k_cache);
+  else
+    latent_prep_kernel<bf16_t><<<grid, 256, 0, st>>>(q_latent, q_rank, (const bf16_t*)q_norm_w, (bf16_t*)q_bf16,
+                                                     ld_q_bf16, kv, kv_rank, rot_dim, (const bf16_t*)kv_norm_w, ld, eps, 1,
+                                                     rot_dims, rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
+                                                     max_blocks, page, (bf16_t*)k_cache);
+  SD_CHECK_LAUNCH("sd_latent_prep");
+  return SD_OK;
+}
+
+extern "C" int sd_qk_norm_append(float* q, int n_q, const void* q_norm_w, float* k, int G, int dk, const void* k_norm_w,
+                                 const float* v, int dv, int64_t ld, int w_f32, float eps, void* k_cache, void* v_cache,
+                                 const int32_t* row_pos, const int32_t* row_slot, const int32_t* block_tables,
+                                 int max_blocks, int page, int n_rows, sd_stream_t stream) {
+  SD_REQUIRE(q && q_norm_w && k && k_norm_w && v && k_cache && v_cache && row_pos && row_slot && block_tables,
+             SD_ERR_INVALID, "sd_qk_norm_append: null argument");
+  SD_REQUIRE(n_rows >= 1 && n_q >= 1 && G >= 1 && dk >= 1 && dv >= 1 && page >= 1 && max_blocks >= 1, SD_ERR_INVALID,
+             "sd_qk_norm_append: bad shape");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, 2);
+  if (w_f32)
+    qk_norm_append_kernel<float><<<grid, 256, 0, st>>>(q, n_q, (const float*)q_norm_w, k, G, dk, (const float*)k_norm_w, v,
+                                                       dv, ld, eps, row_pos, row_slot, block_tables, max_blocks, page,
+                                                       (float*)k_cache, (float*)v_cache);
+  else
+    qk_norm_append_kernel<bf16_t><<<grid, 256, 0, st>>>(q, n_q, (const bf16_t*)q_norm_w, k, G, dk, (const bf16_t*)k_norm_w,
+                                                        v, dv, ld, eps, row_pos, row_slot, block_tables, max_blocks, page,
+                                                        (bf16_t*)k_cache, (bf16_t*)v_cache);
+  SD_CHECK_LAUNCH("sd_qk_norm_append");
+  return SD_OK;
 }
 
 extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, void* k_cache, void* v_cache,

@@ -1504,6 +1504,12 @@ extern "C" int sd_rope_rows(float*, int64_t, const int32_t*, int, int, int, int,
                             sd_stream_t) { UNSUPPORTED("sd_rope_rows"); }
 extern "C" int sd_rope_copy_rows(const float*, int64_t, int, int, float*, int64_t, int, int, const int32_t*, int, int,
                                  int, int, int, const double*, float, sd_stream_t) { UNSUPPORTED("sd_rope_copy_rows"); }
+extern "C" int sd_latent_prep(float*, int, const void*, void*, int64_t, float*, int, int, const void*, int64_t, int,
+                              float, int, int, const double*, float, void*, const int32_t*, const int32_t*,
+                              const int32_t*, int, int, int, sd_stream_t) { UNSUPPORTED("sd_latent_prep"); }
+extern "C" int sd_qk_norm_append(float*, int, const void*, float*, int, int, const void*, const float*, int, int64_t,
+                                 int, float, void*, void*, const int32_t*, const int32_t*, const int32_t*, int, int,
+                                 int, sd_stream_t) { UNSUPPORTED("sd_qk_norm_append"); }
 extern "C" int sd_cache_append(const float*, int64_t, const float*, int64_t, void*, void*, int, const int32_t*,
                                const int32_t*, const int32_t*, int, int, int, int, int, int, sd_stream_t) {
   UNSUPPORTED("sd_cache_append");

@@ -1343,3 +1343,38 @@ def postnorm_residual(x, a, w, eps, n_a=1, sa=1.0, b=None, sb=0.0) -> None:
     _lib.check(_lib.load().sd_postnorm_residual(_p(x), _p(a), int(n_a), float(sa), _p(b), float(sb), _p(w),
                                                 _wkind(w, "w"), float(eps), None, x.shape[0], x.shape[1], _stream()),
                "sd_postnorm_residual")
+
+
+def latent_prep(q_latent, q_norm_w, kv, kv_norm_w, kv_rank, rot_dim, eps, rot_dims, inv_freq, mag, k_cache,
+                row_pos, row_slot, block_tables, layout=1) -> None:
+    """In place on q_latent f32 [rows, q_rank] and kv f32 [rows, kv_rank + rot_dim]; appends the
+    finished kv rows to k_cache [pages, 1, PAGE, kv_rank + rot_dim].  See sd_latent_prep."""
+    _f32(q_latent, "q_latent")
+    _f32(kv, "kv")
+    n = kv.shape[0]
+    buf = torch.cat([q_latent, kv], dim=1).contiguous()      # the entry point takes one row stride
+    qr = q_latent.shape[1]
+    _lib.check(_lib.load().sd_latent_prep(buf.data_ptr(), qr, _p(q_norm_w), None, 0, buf.data_ptr() + 4 * qr, kv_rank,
+                                          rot_dim, _p(kv_norm_w), buf.shape[1], _wkind(q_norm_w, "q_norm_w"),
+                                          float(eps), rot_dims, layout, _p(inv_freq), float(mag), _p(k_cache),
+                                          _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, n,
+                                          _stream()), "sd_latent_prep")
+    q_latent.copy_(buf[:, :qr])
+    kv.copy_(buf[:, qr:])
+
+
+def qk_norm_append(q, q_norm_w, k, k_norm_w, v, G, dk, dv, eps, k_cache, v_cache, row_pos, row_slot,
+                   block_tables) -> None:
+    """In place on q f32 [rows, n_q] and k f32 [rows, G*dk] (each normed over all its columns);
+    appends k and v f32 [rows, G*dv] to the caches.  See sd_qk_norm_append."""
+    for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+        _f32(t, nm)
+    buf = torch.cat([q, k, v], dim=1).contiguous()
+    nq, nk = q.shape[1], k.shape[1]
+    _lib.check(_lib.load().sd_qk_norm_append(buf.data_ptr(), nq, _p(q_norm_w), buf.data_ptr() + 4 * nq, G, dk,
+                                             _p(k_norm_w), buf.data_ptr() + 4 * (nq + nk), dv, buf.shape[1],
+                                             _wkind(q_norm_w, "q_norm_w"), float(eps), _p(k_cache), _p(v_cache),
+                                             _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE,
+                                             q.shape[0], _stream()), "sd_qk_norm_append")
+    q.copy_(buf[:, :nq])
+    k.copy_(buf[:, nq:nq + nk])
