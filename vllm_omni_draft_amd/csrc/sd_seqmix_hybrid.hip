@@ -1146,6 +1146,103 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
     }
 }
 
+// ---- a few assignments (decoding): each is a matrix-vector product.  A workgroup holds the
+// assignment's input row in LDS; a wave owns a few output columns, its lanes stride over k in
+// 16-byte pieces of the weight rows (a row is read in whole coalesced lines, all of a wave's
+// loads asked for before the first is used), then a butterfly sum.
+constexpr int kGemvMaxK = 8192;
+// act[a, n] (bf16) = silu(s * gate_e[n] . x) * (s * up_e[n] . x); wave: two columns, gate and up.
+__global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
+    const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ sel_e, const float* __restrict__ sel_w,
+    const bf16_t* __restrict__ Wgu, bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
+  extern __shared__ float xs[];   // [K]
+  const int a = blockIdx.y, e = sel_e[a], tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const float* xr = X + (size_t)(a / top) * ldx;
+  for (int k = tid; k < K; k += 256) xs[k] = round_bf16(xr[k]);
+  __syncthreads();
+  const int n0 = blockIdx.x * 8 + wave * 2;
+  if (n0 >= F) return;
+  const int n1 = n0 + 1 < F ? n0 + 1 : n0;
+  const bf16_t* wg = Wgu + (size_t)e * 2 * F * K;
+  const bf16_t* wu = wg + (size_t)F * K;
+  const bf16_t* rows[4] = {wg + (size_t)n0 * K, wu + (size_t)n0 * K, wg + (size_t)n1 * K, wu + (size_t)n1 * K};
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = lane * 8; k0 < K; k0 += 4 * 512) {
+    bf16x8 f[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 512 * u < K ? k0 + 512 * u : k0;   // unguarded, on an address inside the row
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[u][j] = *reinterpret_cast<const bf16x8*>(rows[j] + k);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 512 * u;
+      if (k < K) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xv = xs[k + i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] = fmaf(xv, (float)f[u][j][i], acc[j]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = wave_sum(acc[j]);
+  if (lane == 0) {
+    const float sc = scale_input ? sel_w[a] : 1.f;
+    act[(size_t)a * F + n0] = (bf16_t)(silu_f(sc * acc[0]) * (sc * acc[1]));
+    if (n0 + 1 < F) act[(size_t)a * F + n0 + 1] = (bf16_t)(silu_f(sc * acc[2]) * (sc * acc[3]));
+  }
+}
+
+// out[a, n] = down_e[n] . act[a]; wave: four columns.
+__global__ __launch_bounds__(256) void moe_gemv_down_kernel(
+    const bf16_t* __restrict__ act, const int32_t* __restrict__ sel_e, const float* __restrict__ sel_w,
+    const bf16_t* __restrict__ Wd, float* __restrict__ out, int N, int K, int scale_input) {
+  extern __shared__ float xs[];   // [K]
+  const int a = blockIdx.y, e = sel_e[a], tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (int k = tid; k < K; k += 256) xs[k] = (float)act[(size_t)a * K + k];
+  __syncthreads();
+  const int n0 = blockIdx.x * 16 + wave * 4;
+  if (n0 >= N) return;
+  const bf16_t* w = Wd + (size_t)e * N * K;
+  const bf16_t* rows[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rows[j] = w + (size_t)(n0 + j < N ? n0 + j : n0) * K;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = lane * 8; k0 < K; k0 += 4 * 512) {
+    bf16x8 f[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 512 * u < K ? k0 + 512 * u : k0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[u][j] = *reinterpret_cast<const bf16x8*>(rows[j] + k);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 512 * u;
+      if (k < K) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xv = xs[k + i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] = fmaf(xv, (float)f[u][j][i], acc[j]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = wave_sum(acc[j]);
+  if (lane == 0) {
+    const float sc = scale_input ? 1.f : sel_w[a];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n0 + j < N) out[(size_t)a * N + n0 + j] = sc * acc[j];
+  }
+}
+
 struct MoeScratch {
   size_t cnt, n_tiles, perm, tiles, act, total;
 };
@@ -1541,6 +1638,14 @@ extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, c
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_kernel<float><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
                                                                          (const float*)w_down, out, W, F, scale_input);
+  } else if (!tiles && W % 8 == 0 && F % 8 == 0 && W <= kGemvMaxK && F <= kGemvMaxK && sd_aligned16(w_gate_up) &&
+             sd_aligned16(w_down)) {
+    bf16_t* act_b = (bf16_t*)act;
+    moe_gemv_gate_up_kernel<<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
+        x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
+    SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
+    moe_gemv_down_kernel<<<dim3((W + 15) / 16, n), 256, sizeof(float) * F, st>>>(
+        act_b, sel_expert, sel_weight, (const bf16_t*)w_down, out, W, F, scale_input);
   } else if (mfma) {
     // (act holds n * F floats: its first half serves as the bf16 activations)
     bf16_t* act_b = (bf16_t*)act;
